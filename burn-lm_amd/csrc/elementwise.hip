@@ -8,22 +8,27 @@
 // ---------------------------------------------------------------------------------------
 template <typename TW>
 __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ h, int D) {
+                                    float* __restrict__ h, int D, int copies) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const TW* row = table + (size_t)id * D;
-  float* out = h + (size_t)t * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = to_float(row[d]);
+  float* out = h + (size_t)t * copies * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = to_float(row[d]);
+    for (int c = 0; c < copies; ++c) out[(size_t)c * D + d] = v;
+  }
 }
 
+// copies: h is [T][copies][D] and every copy of a token's row is the same (residual arrangements with
+// several streams start from equal streams)
 extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* ids, float* h,
-                                int T, int D, hipStream_t stream) {
-  BLM_REQUIRE(T > 0 && D > 0, "embed_gather: bad sizes T=%d D=%d", T, D);
+                                int T, int D, int copies, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0 && copies >= 1, "embed_gather: bad sizes T=%d D=%d copies=%d", T, D, copies);
   dim3 grid(T), block(256);
   if (table_dtype == BLM_F32)
-    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, (const float*)table, ids, h, D);
+    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, (const float*)table, ids, h, D, copies);
   else if (table_dtype == BLM_BF16)
-    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, h, D);
+    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, h, D, copies);
   else
     return blm_fail("embed_gather: unsupported table dtype %d", table_dtype);
   BLM_LAUNCH_CHECK("embed_gather");
@@ -37,32 +42,35 @@ extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* i
 template <typename TW>
 __global__ void embed_gather_from_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
                                          const int* __restrict__ source_rows, const int* const* __restrict__ source,
-                                         float* __restrict__ h, int D, int V) {
+                                         float* __restrict__ h, int D, int V, int copies) {
   const int t = blockIdx.x;
   const int r = source_rows[t];
   const int id = r >= 0 ? (*source)[r] : ids[t];
-  float* out = h + (size_t)t * D;
+  float* out = h + (size_t)t * copies * D;
   if ((unsigned)id >= (unsigned)V) {
-    for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = __builtin_nanf("");
+    for (int d = threadIdx.x; d < copies * D; d += blockDim.x) out[d] = __builtin_nanf("");
     return;
   }
   const TW* row = table + (size_t)id * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) out[d] = to_float(row[d]);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    const float v = to_float(row[d]);
+    for (int c = 0; c < copies; ++c) out[(size_t)c * D + d] = v;
+  }
 }
 
 extern "C" int blm_embed_gather_from(const void* table, int table_dtype, const int* ids, const int* source_rows,
-                                     const void* source_cell, float* h, int T, int D, int V, hipStream_t stream) {
-  BLM_REQUIRE(T > 0 && D > 0 && V > 0, "embed_gather_from: bad sizes T=%d D=%d V=%d", T, D, V);
+                                     const void* source_cell, float* h, int T, int D, int V, int copies, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0 && V > 0 && copies >= 1, "embed_gather_from: bad sizes T=%d D=%d V=%d", T, D, V);
   BLM_REQUIRE(source_rows && source_cell && ((size_t)source_cell & 7) == 0,
               "embed_gather_from: needs the rows and an 8-byte aligned cell with the tokens' address");
   dim3 grid(T), block(256);
   const int* const* cell = (const int* const*)source_cell;
   if (table_dtype == BLM_F32)
     hipLaunchKernelGGL(embed_gather_from_kernel<float>, grid, block, 0, stream, (const float*)table, ids, source_rows,
-                       cell, h, D, V);
+                       cell, h, D, V, copies);
   else if (table_dtype == BLM_BF16)
     hipLaunchKernelGGL(embed_gather_from_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, source_rows,
-                       cell, h, D, V);
+                       cell, h, D, V, copies);
   else
     return blm_fail("embed_gather_from: unsupported table dtype %d", table_dtype);
   BLM_LAUNCH_CHECK("embed_gather_from");

@@ -1,0 +1,336 @@
+// Attention over a shared low-rank latent (one cached row per token for all heads).
+//
+// A token's cache row is [latent c (R lanes) | rotated key part (Dr lanes)]; the key page layout is that
+// of every other attention of this library with one key head of R + Dr lanes, and there are no value
+// pages: the values are the latent lanes of the same rows.  Queries come "absorbed": per head
+// [W_uk^T q_plain (R lanes) | rotated query part (Dr lanes)] in float, so a score is one dot product of
+// R + Dr lanes against the cache row, and a head's result is the probability-weighted sum of latents
+// (R lanes), which the caller expands with W_uv.
+//
+// Kernels: the write of a step's tokens into the cache (RMS norm of the latent, rotation of the shared
+// key part and of the queries' rotated parts), a small batched product per head, and the attention.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// down [T][ld_down]: R latent lanes then Dr key lanes.  q [T][ld_q], head h at h * (dn + Dr).  cos_sin [positions][half_t]
+// (cos, sin), of which the first rot/2 pairs turn lanes (i, i + rot/2) of the Dr part.
+// qabs [T][H][R + Dr] float gets the rotated query parts at lane R.
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, const TA* __restrict__ q, int ld_q, int H, int dn,
+                                    const float* __restrict__ norm_w, float eps, const float2* __restrict__ cos_sin,
+                                    int half_t, int rot, float* __restrict__ qabs, TA* __restrict__ kcache,
+                                    const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                    const int* __restrict__ block_table, int table_width, int page_size, int R, int Dr,
+                                    int write_kv) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const int b = token_seq[t];
+  if (b < 0) return;
+  const int pos = positions[t];
+  const float2* cs = cos_sin + (size_t)pos * half_t;
+  const int half = rot >> 1;
+  // queries: rotated parts into the absorbed rows
+  for (int i = threadIdx.x; i < H * Dr; i += blockDim.x) {
+    const int h = i / Dr, d = i - h * Dr;
+    const TA* src = q + (size_t)t * ld_q + (size_t)h * (dn + Dr) + dn;
+    float v = to_float(src[d]);
+    if (d < rot) {
+      const int pair = d < half ? d : d - half;
+      const float2 c = cs[pair];
+      const float other = to_float(src[d < half ? d + half : d - half]);
+      v = d < half ? v * c.x - other * c.y : v * c.x + other * c.y;
+    }
+    qabs[((size_t)t * H + h) * (R + Dr) + R + d] = v;
+  }
+  const int page = block_table[(size_t)b * table_width + pos / page_size];
+  if (!write_kv || page < 0) return;
+  const TA* row = down + (size_t)t * ld_down;
+  TA* dst = kcache + ((size_t)page * page_size + (pos % page_size)) * (R + Dr);
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    const float v = to_float(row[d]);
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum<true>(ss, red) / (float)R + eps);
+  for (int d = threadIdx.x; d < R; d += blockDim.x) dst[d] = from_float<TA>(to_float(row[d]) * inv * norm_w[d]);
+  for (int d = threadIdx.x; d < Dr; d += blockDim.x) {
+    float v = to_float(row[R + d]);
+    if (d < rot) {
+      const int pair = d < half ? d : d - half;
+      const float2 c = cs[pair];
+      const float other = to_float(row[R + (d < half ? d + half : d - half)]);
+      v = d < half ? v * c.x - other * c.y : v * c.x + other * c.y;
+    }
+    dst[R + d] = from_float<TA>(v);
+  }
+}
+
+extern "C" int blm_latent_write(const void* down, int ld_down, const void* q, int ld_q, int dtype, int T, int H, int dn,
+                                const float* norm_w, float eps, const void* cos_sin, int half_t, int rot, float* qabs,
+                                void* kcache, const int* positions, const int* token_seq, const int* block_table,
+                                int table_width, int page_size, int R, int Dr, int write_kv, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && H > 0 && dn >= 0 && R > 0 && Dr >= 0, "latent_write: bad sizes");
+  BLM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= Dr && rot / 2 <= half_t, "latent_write: %d turning lanes do not fit %d", rot, Dr);
+  BLM_REQUIRE(page_size > 0 && table_width > 0 && ld_down >= R + Dr && ld_q >= H * (dn + Dr), "latent_write: bad geometry");
+#define BLM_LW(TA)                                                                                                      \
+  hipLaunchKernelGGL(latent_write_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)down, ld_down, (const TA*)q, ld_q, H, \
+                     dn, norm_w, eps, (const float2*)cos_sin, half_t, rot, qabs, (TA*)kcache, positions, token_seq,     \
+                     block_table, table_width, page_size, R, Dr, write_kv)
+  if (dtype == BLM_F32) BLM_LW(float);
+  else if (dtype == BLM_BF16) BLM_LW(bf16);
+  else return blm_fail("latent_write: unsupported dtype %d", dtype);
+#undef BLM_LW
+  BLM_LAUNCH_CHECK("latent_write");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Batched product per head: out[t][h][n] = sum_k in[t][h][k] * w[h][n][k], float accumulation.
+// in: rows of `in_row` elements, head h at h * in_head; out likewise; w [H][N][K] contiguous.
+// 64 x 64 tile per block of 256 threads, 16 of K per stage in shared memory, 4 x 4 results per thread.
+// ---------------------------------------------------------------------------------------
+#define HP_TILE 64
+#define HP_K 16
+template <typename TI, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+    head_project_kernel(const TI* __restrict__ in, long long in_row, int in_head, const TW* __restrict__ w,
+                        TO* __restrict__ out, long long out_row, int out_head, int T, int N, int K) {
+  __shared__ float sa[HP_K][HP_TILE + 1], sb[HP_K][HP_TILE + 1];
+  const int h = blockIdx.z;
+  const int t0 = blockIdx.x * HP_TILE, n0 = blockIdx.y * HP_TILE;
+  const TI* a = in + (size_t)h * in_head;
+  const TW* bw = w + (size_t)h * N * K;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += HP_K) {
+    for (int i = threadIdx.x; i < HP_TILE * HP_K; i += 256) {
+      const int r = i / HP_K, k = i - r * HP_K;
+      const int t = t0 + r, n = n0 + r, kk = k0 + k;
+      sa[k][r] = (t < T && kk < K) ? to_float(a[(size_t)t * in_row + kk]) : 0.f;
+      sb[k][r] = (n < N && kk < K) ? to_float(bw[(size_t)n * K + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < HP_K; ++k) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = sa[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = sb[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = t0 + ty * 4 + i;
+    if (t >= T) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) out[(size_t)t * out_row + (size_t)h * out_head + n] = from_float<TO>(acc[i][j]);
+    }
+  }
+}
+
+extern "C" int blm_head_project(const void* in, int in_dtype, long long in_row, int in_head, const void* w, int w_dtype,
+                                void* out, int out_dtype, long long out_row, int out_head, int T, int H, int N, int K,
+                                hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && H > 0 && N > 0 && K > 0 && H <= 65535, "head_project: bad sizes T=%d H=%d N=%d K=%d", T, H, N, K);
+  dim3 grid((T + HP_TILE - 1) / HP_TILE, (N + HP_TILE - 1) / HP_TILE, H), block(256);
+  BLM_REQUIRE(grid.y <= 65535, "head_project: too many columns");
+#define BLM_HP(TI, TW, TO)                                                                                       \
+  hipLaunchKernelGGL((head_project_kernel<TI, TW, TO>), grid, block, 0, stream, (const TI*)in, in_row, in_head,  \
+                     (const TW*)w, (TO*)out, out_row, out_head, T, N, K)
+  if (in_dtype == BLM_F32 && w_dtype == BLM_F32 && out_dtype == BLM_F32) BLM_HP(float, float, float);
+  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) BLM_HP(bf16, bf16, float);
+  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) BLM_HP(float, bf16, bf16);
+  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) BLM_HP(bf16, bf16, bf16);
+  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) BLM_HP(float, bf16, float);
+  else return blm_fail("head_project: unsupported dtypes in=%d w=%d out=%d", in_dtype, w_dtype, out_dtype);
+#undef BLM_HP
+  BLM_LAUNCH_CHECK("head_project");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// The attention, generic form: one wavefront per (query token, head); prompts and decoding alike.
+// Query at position p of its sequence sees rows j <= p of the same sequence.  A chunk of 64 rows at a
+// time: every lane scores one row (R + Dr lanes against the query in shared memory), the running maximum
+// and sum follow, then every lane owns latent lanes lane, lane + 64, ... of the weighted sum and walks the
+// chunk's rows.  With n_splits > 1 the rows of a (token, head) are cut into pieces for different
+// wavefronts, whose partial results the last one to arrive merges (as in the generic attention).
+// olat [T][H][R] float.
+// ---------------------------------------------------------------------------------------
+#define LAT_WAVES 4
+#define LAT_MAX_R 1024
+template <typename TA>
+__global__ void __launch_bounds__(LAT_WAVES* BLM_WAVE)
+    latent_attn_kernel(const float* __restrict__ qabs, float* __restrict__ olat, const int* __restrict__ positions,
+                       const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_width,
+                       const TA* __restrict__ kcache, int page_size, int T, int H, int R, int Dr, float scale,
+                       int n_splits, float* part_o, float* part_ml, int* arrivals) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int W = R + Dr;
+  const long long item = (long long)blockIdx.x * LAT_WAVES + wave;
+  const bool active = item < (long long)T * H;
+  const int t = active ? (int)(item / H) : 0;
+  const int b = active ? token_seq[t] : -1;
+  float* qs = smem + (size_t)wave * W;
+  if (active && b >= 0) {
+    const float* qrow = qabs + (size_t)item * W;
+    for (int d = lane; d < W; d += BLM_WAVE) qs[d] = qrow[d];
+  }
+  __syncthreads();
+  if (!active) return;
+  float* orow = olat + (size_t)item * R;
+  if (b < 0) {
+    for (int d = lane; d < R; d += BLM_WAVE) orow[d] = 0.f;
+    return;
+  }
+  const int pos = positions[t];
+  const int* bt = block_table + (size_t)b * table_width;
+  const int split = blockIdx.y;
+  const int n_chunks = pos / BLM_WAVE + 1;
+  const int per_split = (n_chunks + n_splits - 1) / n_splits;
+  const int j_begin = split * per_split * BLM_WAVE;
+  const int j_end = min(pos, j_begin + per_split * BLM_WAVE - 1);
+
+  float m = -INFINITY, l = 0.f;
+  float acc[LAT_MAX_R / BLM_WAVE];
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) acc[i] = 0.f;
+  const bool vec = (W % 8) == 0;
+
+  for (int j0 = j_begin; j0 <= j_end; j0 += BLM_WAVE) {
+    const int j = j0 + lane;
+    const bool valid = j <= j_end;
+    float s = -INFINITY;
+    if (valid) {
+      const int page = bt[j / page_size];
+      const TA* krow = kcache + ((size_t)page * page_size + (j % page_size)) * W;
+      float dot = 0.f;
+      if (vec && sizeof(TA) == 2) {
+        for (int d = 0; d < W; d += 8) {
+          const uint4 raw = *reinterpret_cast<const uint4*>(krow + d);
+          const uint32_t ws[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            dot = fmaf(qs[d + 2 * i], __uint_as_float(ws[i] << 16), dot);
+            dot = fmaf(qs[d + 2 * i + 1], __uint_as_float(ws[i] & 0xffff0000u), dot);
+          }
+        }
+      } else {
+        for (int d = 0; d < W; ++d) dot = fmaf(qs[d], to_float(krow[d]), dot);
+      }
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float corr = expf(m - m_new);
+    l = l * corr + wave_sum(p);
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) acc[i] *= corr;
+    const int cnt = (j_end - j0 + 1) < BLM_WAVE ? (j_end - j0 + 1) : BLM_WAVE;
+    for (int jj = 0; jj < cnt; ++jj) {
+      const float pj = __shfl(p, jj, BLM_WAVE);
+      const int ja = j0 + jj;
+      const int page = bt[ja / page_size];
+      const TA* crow = kcache + ((size_t)page * page_size + (ja % page_size)) * W;
+#pragma unroll
+      for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) {
+        const int d = lane + i * BLM_WAVE;
+        if (d < R) acc[i] = fmaf(pj, to_float(crow[d]), acc[i]);
+      }
+    }
+    m = m_new;
+  }
+  if (n_splits == 1) {
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) {
+      const int d = lane + i * BLM_WAVE;
+      if (d < R) orow[d] = acc[i] * inv;
+    }
+    return;
+  }
+  float* po = part_o + ((size_t)item * n_splits + split) * R;
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) {
+    const int d = lane + i * BLM_WAVE;
+    if (d < R) __hip_atomic_store(po + d, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (lane == 0) {
+    __hip_atomic_store(part_ml + ((size_t)item * n_splits + split) * 2, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part_ml + ((size_t)item * n_splits + split) * 2 + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the wavefront's stores have been acknowledged
+  int last = 0;
+  if (lane == 0) {
+    const int before = __hip_atomic_fetch_add(arrivals + item, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = before == n_splits - 1;
+    if (last) __hip_atomic_store(arrivals + item, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  last = __shfl(last, 0, BLM_WAVE);
+  if (!last) return;
+  float M = -INFINITY, L = 0.f;
+  float O[LAT_MAX_R / BLM_WAVE];
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) O[i] = 0.f;
+  for (int sp = 0; sp < n_splits; ++sp) {
+    const float* ml = part_ml + ((size_t)item * n_splits + sp) * 2;
+    const float ms = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float ls = __hip_atomic_load(ml + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ls == 0.f) continue;
+    const float Mn = fmaxf(M, ms);
+    const float keep = expf(M - Mn), take = expf(ms - Mn);
+    L = L * keep + ls * take;
+    const float* ps = part_o + ((size_t)item * n_splits + sp) * R;
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) {
+      const int d = lane + i * BLM_WAVE;
+      if (d < R) O[i] = O[i] * keep + __hip_atomic_load(ps + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * take;
+    }
+    M = Mn;
+  }
+  const float inv = 1.0f / L;
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_R / BLM_WAVE; ++i) {
+    const int d = lane + i * BLM_WAVE;
+    if (d < R) orow[d] = O[i] * inv;
+  }
+}
+
+// part_o: T*H*n_splits*R floats, part_ml: T*H*n_splits*2 floats, arrivals: T*H ints, zero before the
+// first call and left zero; all three may be null when n_splits is 1.
+extern "C" int blm_latent_attn(const float* qabs, float* olat, int cache_dtype, const int* positions,
+                               const int* token_seq, const int* block_table, int table_width, const void* kcache,
+                               int page_size, int T, int H, int R, int Dr, float scale, int n_splits, float* part_o,
+                               float* part_ml, int* arrivals, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && H > 0 && R > 0 && Dr >= 0, "latent_attn: bad sizes T=%d H=%d R=%d Dr=%d", T, H, R, Dr);
+  BLM_REQUIRE(R <= LAT_MAX_R, "latent_attn: a latent of %d lanes is more than %d", R, LAT_MAX_R);
+  BLM_REQUIRE(page_size > 0 && table_width > 0, "latent_attn: bad cache geometry");
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml && arrivals)),
+              "latent_attn: %d splits need their workspace", n_splits);
+  const long long items = (long long)T * H;
+  const long long blocks = (items + LAT_WAVES - 1) / LAT_WAVES;
+  BLM_REQUIRE(blocks < 2147483647LL, "latent_attn: too many (token, head) pairs");
+  const size_t smem = (size_t)LAT_WAVES * (R + Dr) * sizeof(float);
+  BLM_REQUIRE(smem <= 64 * 1024, "latent_attn: query rows of %d lanes do not fit shared memory", R + Dr);
+  dim3 grid((unsigned)blocks, (unsigned)n_splits), block(LAT_WAVES * BLM_WAVE);
+  if (cache_dtype == BLM_F32)
+    hipLaunchKernelGGL(latent_attn_kernel<float>, grid, block, smem, stream, qabs, olat, positions, token_seq, block_table,
+                       table_width, (const float*)kcache, page_size, T, H, R, Dr, scale, n_splits, part_o, part_ml, arrivals);
+  else if (cache_dtype == BLM_BF16)
+    hipLaunchKernelGGL(latent_attn_kernel<bf16>, grid, block, smem, stream, qabs, olat, positions, token_seq, block_table,
+                       table_width, (const bf16*)kcache, page_size, T, H, R, Dr, scale, n_splits, part_o, part_ml, arrivals);
+  else
+    return blm_fail("latent_attn: unsupported dtype %d", cache_dtype);
+  BLM_LAUNCH_CHECK("latent_attn");
+  return 0;
+}

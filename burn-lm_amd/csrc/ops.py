@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 _lib = None
 _lock = threading.Lock()
 
@@ -22,9 +22,29 @@ class KernelError(RuntimeError):
 
 
 _SIGNATURES = {
-    "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "blm_embed_gather_from": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                              _c_void_p],
+                              _c_int, _c_void_p],
+    "blm_streams_norm": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_void_p, _c_void_p,
+                         _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_float,
+                         _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+    "blm_token_shift": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                        _c_int, _c_int, _c_void_p],
+    "blm_xielu": [_c_void_p, _c_void_p, _c_int, ctypes.c_longlong, _c_float, _c_float, _c_void_p],
+    "blm_latent_write": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_void_p,
+                         _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                         _c_int, _c_int, _c_void_p],
+    "blm_head_project": [_c_void_p, _c_int, ctypes.c_longlong, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
+                         ctypes.c_longlong, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_latent_attn": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int,
+                        _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+    "blm_hgrn2_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p,
+                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_conv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                         _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_delta_scan": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                       _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_void_p],
     "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p, _c_int,
                         _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -183,15 +203,21 @@ def _check_planes(who, kcache, vcache, nkv, page_size, hd):
 
 
 # ------------------------------------------------------------------------------------------
+def _embed_shape(who, table, out_h):
+    """(T, D, copies) of an embedding output [T, D] or [T, copies, D]."""
+    if out_h.dtype != torch.float32 or out_h.dim() not in (2, 3) or table.shape[1] != out_h.shape[-1]:
+        raise KernelError(f"{who}: h must be float32 [T, D] or [T, copies, D] with D the table's width")
+    return out_h.shape[0], out_h.shape[-1], (out_h.shape[1] if out_h.dim() == 3 else 1)
+
+
 def embed_gather(table, ids, out_h):
-    """out_h[t, :] = table[ids[t], :] as float32.  ids must already be checked against the vocabulary."""
+    """out_h[t, :] = table[ids[t], :] as float32 (out_h [T, copies, D]: every copy alike).  ids must already be
+    checked against the vocabulary."""
     _gpu(table, ids, out_h)
-    T, D = out_h.shape
+    T, D, copies = _embed_shape("embed_gather", table, out_h)
     _i32("ids", ids, T)
     _contig("table", table); _contig("h", out_h)
-    if out_h.dtype != torch.float32 or table.shape[1] != D:
-        raise KernelError("embed_gather: h must be float32 [T, D] with D the table's width")
-    _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, _stream())
+    _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, copies, _stream())
     return out_h
 
 
@@ -200,16 +226,14 @@ def embed_gather_from(table, ids, source_rows, source_cell, out_h):
     element source_rows[t] of the int32 array whose address stands in source_cell (an int64 tensor of
     one element on the device).  A token outside the vocabulary gives a row of NaN."""
     _gpu(table, ids, source_rows, source_cell, out_h)
-    T, D = out_h.shape
+    T, D, copies = _embed_shape("embed_gather_from", table, out_h)
     _i32("ids", ids, T)
     _i32("source_rows", source_rows, T)
     _contig("table", table); _contig("h", out_h)
-    if out_h.dtype != torch.float32 or table.shape[1] != D:
-        raise KernelError("embed_gather_from: h must be float32 [T, D] with D the table's width")
     if source_cell.dtype != torch.int64 or source_cell.numel() != 1:
         raise KernelError("embed_gather_from: the cell is one int64 on the device")
     _call("blm_embed_gather_from", table.data_ptr(), _code(table), ids.data_ptr(), source_rows.data_ptr(),
-          source_cell.data_ptr(), out_h.data_ptr(), T, D, table.shape[0], _stream())
+          source_cell.data_ptr(), out_h.data_ptr(), T, D, table.shape[0], copies, _stream())
     return out_h
 
 
@@ -727,3 +751,232 @@ def _probe_sink(device):
     if index not in _sinks:
         _sinks[index] = torch.zeros(4, dtype=torch.float32, device=f"cuda:{index}")
     return _sinks[index]
+
+
+# ------------------------------------------------------------------------------------------
+# residual arrangements with several streams, token shift, xIELU
+def _f32(name, t, n=None):
+    if t.dtype != torch.float32:
+        raise KernelError(f"{name} must be float32, got {t.dtype}")
+    _contig(name, t)
+    if n is not None and t.numel() != n:
+        raise KernelError(f"{name} has {t.numel()} elements, needs {n}")
+
+
+def streams_norm(x, out, gamma, beta, eps, read=None, pending=None, rows=None, write_x=True, out_scale=1.0,
+                 stash=None):
+    """x: float32 streams [T, S, D].  pending: None or (y, scale, mix, write): the result y ([T, D] in bfloat16 or
+    float32, or float32 planes [P, T, D] that are summed) of the sublayer before, still to be written into the
+    streams as ``x'_t = sum_s mix[s, t] x_s + write[t] * y * scale`` (kept if write_x).  Then
+    ``u = sum_t read[t] x'_t`` (read None: the plain sum) and ``out = layer_norm(u; gamma, beta, eps) * out_scale``
+    for every row, or for the rows listed in `rows`.  stash: None or (carry [slots, D], stash [B, D], step): the
+    first token of each of the step's sequences copies its sequence's carry (zeros at position 0) into stash."""
+    _gpu(x, out, gamma, beta, read, rows)
+    if x.dtype != torch.float32 or x.dim() != 3:
+        raise KernelError("streams_norm: the streams are float32 [T, S, D]")
+    T, S, D = x.shape
+    _contig("x", x); _contig("out", out)
+    _f32("gamma", gamma, D); _f32("beta", beta, D)
+    if read is not None:
+        _f32("read", read, S)
+    n_out = out.shape[0]
+    if out.shape[1] != D:
+        raise KernelError(f"streams_norm: out is {tuple(out.shape)}, the width is {D}")
+    y = scale = mix = write = None
+    planes, stride, ycode = 1, 0, 0
+    if pending is not None:
+        y, scale, mix, write = pending
+        _gpu(y, scale, mix, write)
+        _contig("y", y)
+        _f32("scale", scale, D); _f32("mix", mix, S * S); _f32("write", write, S)
+        if y.dim() == 3:
+            if tuple(y.shape[1:]) != (T, D) or y.dtype != torch.float32:
+                raise KernelError("streams_norm: partial results must be float32 [planes, T, D]")
+            planes, stride = y.shape[0], T * D
+        elif tuple(y.shape) != (T, D):
+            raise KernelError(f"streams_norm: the pending result is {tuple(y.shape)}, expected {(T, D)}")
+        ycode = _code(y)
+    if rows is not None:
+        _i32("rows", rows, n_out)
+    elif n_out != T:
+        raise KernelError("streams_norm: out needs one row per token when rows is not given")
+    carry = stash_buf = step = None
+    if stash is not None:
+        carry, stash_buf, step = stash
+        _f32("carry", carry); _f32("stash", stash_buf)
+        if carry.shape[-1] != D or stash_buf.shape != (step.n_seqs, D) or rows is not None:
+            raise KernelError("streams_norm: the stash is [sequences, D], the carry [slots, D], and all rows run")
+    _call("blm_streams_norm", x.data_ptr(), S, _ptr(y), ycode, planes, stride, _ptr(scale), _ptr(mix), _ptr(write),
+          _ptr(read), gamma.data_ptr(), beta.data_ptr(), out.data_ptr(), _code(out), _ptr(rows), n_out, D, float(eps),
+          float(out_scale), 1 if write_x else 0, _ptr(carry), _ptr(stash_buf),
+          step.token_seq.data_ptr() if step else 0, step.cu_seqlens.data_ptr() if step else 0,
+          step.seq_slots.data_ptr() if step else 0, step.positions.data_ptr() if step else 0, _stream())
+    return out
+
+
+def token_shift(n, mu, stash, carry, out, step):
+    """out[t] = n[t] + (prev - n[t]) * mu with prev = n[t - 1] inside a sequence's tokens of this step and
+    stash[sequence] for its first; the last token of a sequence leaves n[t] in carry[slot]."""
+    _gpu(n, mu, stash, carry, out)
+    T, D = n.shape
+    _f32("n", n); _f32("mu", mu, D); _f32("stash", stash, step.n_seqs * D); _f32("carry", carry)
+    _contig("out", out)
+    if tuple(out.shape) != (T, D) or carry.shape[-1] != D or T != step.n_tokens:
+        raise KernelError("token_shift: shapes do not fit")
+    _call("blm_token_shift", n.data_ptr(), mu.data_ptr(), stash.data_ptr(), carry.data_ptr(), out.data_ptr(), _code(out),
+          step.token_seq.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, D, _stream())
+    return out
+
+
+def xielu(z, out, a_pos, a_neg):
+    """z > 0: a_pos z^2 + z/2; else a_neg (exp(z) - 1 - z) + z/2, element by element."""
+    _gpu(z, out)
+    _contig("z", z); _contig("out", out)
+    if z.shape != out.shape or z.dtype != out.dtype:
+        raise KernelError("xielu: input and output must agree in shape and dtype")
+    _call("blm_xielu", z.data_ptr(), out.data_ptr(), _code(z), z.numel(), float(a_pos), float(a_neg), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# attention over a shared latent
+def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_table, page_size, H, dn, R, Dr,
+                 write_kv=True):
+    """down [T, >= R + Dr]: latent lanes then the shared key lanes; q [T, H * (dn + Dr)].  The latent is RMS-normed
+    (norm_w, eps), the first `rot` of the Dr key lanes are turned by the token's position (pairs half of rot
+    apart; cos_sin float32 [positions, n, 2]), and the row [latent | key lanes] goes into the token's place of the
+    key pages [pages, 1, page, R + Dr].  The queries' Dr lanes are turned alike into qabs[:, :, R:] (float32
+    [T, H, R + Dr])."""
+    _gpu(down, q, norm_w, cos_sin, qabs, kcache, block_table)
+    T = down.shape[0]
+    _contig("cos_sin", cos_sin); _contig("kcache", kcache); _contig("qabs", qabs)
+    _f32("norm_w", norm_w, R); _f32("qabs", qabs, T * H * (R + Dr))
+    if down.stride(1) != 1 or q.stride(1) != 1 or down.dtype != q.dtype or kcache.dtype != q.dtype:
+        raise KernelError("latent_write: down, q and the cache must share a dtype, rows contiguous")
+    if tuple(q.shape) != (T, H * (dn + Dr)) or tuple(kcache.shape[1:]) != (1, page_size, R + Dr):
+        raise KernelError(f"latent_write: q {tuple(q.shape)} / key pages {tuple(kcache.shape)} do not fit")
+    if cos_sin.dtype != torch.float32 or cos_sin.dim() != 3 or cos_sin.shape[2] != 2 or cos_sin.shape[0] <= step.max_position:
+        raise KernelError("latent_write: cos_sin must be float32 [positions, pairs, 2] and cover the step's positions")
+    _i32("block_table", block_table)
+    _call("blm_latent_write", down.data_ptr(), down.stride(0), q.data_ptr(), q.stride(0), _code(q), T, H, dn, norm_w.data_ptr(),
+          float(eps), cos_sin.data_ptr(), cos_sin.shape[1], rot, qabs.data_ptr(), kcache.data_ptr(),
+          step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+          R, Dr, 1 if write_kv else 0, _stream())
+
+
+def head_project(x, in_head, w, out, out_head, K=None):
+    """out[t, h * out_head + n] = sum_k x[t, h * in_head + k] * w[h, n, k] for k < K (default in_head), float
+    accumulation.  x, out: 2-D with contiguous rows (any row stride); w [H, N, K] contiguous."""
+    _gpu(x, w, out)
+    _contig("w", w)
+    H, N, Kw = w.shape
+    K = Kw if K is None else K
+    if K != Kw or x.stride(1) != 1 or out.stride(1) != 1 or x.shape[0] != out.shape[0]:
+        raise KernelError("head_project: shapes do not fit")
+    if (H - 1) * in_head + K > x.shape[1] or (H - 1) * out_head + N > out.shape[1]:
+        raise KernelError("head_project: heads reach past the rows")
+    _call("blm_head_project", x.data_ptr(), _code(x), x.stride(0), in_head, w.data_ptr(), _code(w), out.data_ptr(),
+          _code(out), out.stride(0), out_head, x.shape[0], H, N, K, _stream())
+    return out
+
+
+_latent_scratch = {}
+LATENT_SCRATCH_FLOATS = 1 << 22
+
+
+def latent_attn_init(device):
+    """The workspace of the split form (partial results of the pieces), one per device and of a fixed size, so
+    that a recorded launch's address stays good.  The first call for a device must come before any recording."""
+    device = torch.device(device)
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    buf = _latent_scratch.get(key)
+    if buf is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("latent_attn_init: the first call for a device must come before any graph capture")
+        buf = _latent_scratch[key] = torch.empty(LATENT_SCRATCH_FLOATS, dtype=torch.float32, device=torch.device("cuda", key))
+    return buf
+
+
+def latent_attn_max_splits(T, H, R):
+    """Most pieces a (token, head)'s rows can be cut into for T tokens."""
+    if T * H > ARRIVAL_COUNTERS:
+        return 1
+    return max(1, LATENT_SCRATCH_FLOATS // (T * H * (R + 2)))
+
+
+
+def latent_attn(qabs, olat, kcache, step, block_table, page_size, H, R, Dr, scale, n_splits=1):
+    """softmax over each query's visible rows of (qabs . [latent | key lanes]) * scale, times the latents:
+    olat float32 [T, H, R].  qabs float32 [T, H, R + Dr]; kcache [pages, 1, page, R + Dr]."""
+    _gpu(qabs, olat, kcache, block_table)
+    T = qabs.shape[0]
+    _f32("qabs", qabs, T * H * (R + Dr)); _f32("olat", olat, T * H * R)
+    _contig("kcache", kcache); _i32("block_table", block_table)
+    if tuple(kcache.shape[1:]) != (1, page_size, R + Dr):
+        raise KernelError(f"latent_attn: key pages {tuple(kcache.shape)} do not fit rows of {R + Dr}")
+    part_o = part_ml = arrivals = None
+    if n_splits > 1:
+        need = T * H * n_splits * (R + 2)
+        if n_splits > latent_attn_max_splits(T, H, R):
+            raise KernelError("latent_attn: more pieces than the workspace holds (see latent_attn_max_splits)")
+        buf = latent_attn_init(qabs.device)
+        part_o, part_ml = buf[: T * H * n_splits * R], buf[T * H * n_splits * R: need]
+        arrivals = arrival_counters(qabs.device)
+    _call("blm_latent_attn", qabs.data_ptr(), olat.data_ptr(), _code(kcache), step.positions.data_ptr(),
+          step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), page_size, T, H, R,
+          Dr, float(scale), n_splits, _ptr(part_o), _ptr(part_ml), _ptr(arrivals), _stream())
+    return olat
+
+
+# ------------------------------------------------------------------------------------------
+# recurrent mixers
+def hgrn2_scan(proj, f_bias, low, norm_w, eps, state, out, step, H, dk, dv):
+    """proj [T, >= 2 H dk + H dv]: queries, forget-gate logits, values.  state float32 [slots, H, dk, dv] is read
+    and left updated for the step's sequences; out [T, H * dv] in proj's dtype."""
+    _gpu(proj, f_bias, low, norm_w, state, out)
+    _f32("f_bias", f_bias, H * dk); _f32("low", low, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
+    _contig("out", out)
+    if proj.stride(1) != 1 or out.dtype != proj.dtype or tuple(out.shape) != (proj.shape[0], H * dv) \
+            or tuple(state.shape[1:]) != (H, dk, dv):
+        raise KernelError("hgrn2_scan: shapes do not fit")
+    _call("blm_hgrn2_scan", proj.data_ptr(), _code(proj), proj.stride(0), f_bias.data_ptr(), low.data_ptr(),
+          norm_w.data_ptr(), float(eps), state.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
+          step.seq_slots.data_ptr(), step.n_seqs, H, dk, dv, _stream())
+    return out
+
+
+def conv_prepare(proj, taps_w, hist, out, step, C, G, dk):
+    """Causal convolution per channel over the first C columns of proj ([q: G dk | k: G dk | v]) with SiLU, unit
+    norms of the q and k heads (q also times dk^-1/2) -> out float32 [T, C]; hist float32 [slots, taps - 1, C] is
+    read and then left holding each sequence's last taps - 1 inputs."""
+    _gpu(proj, taps_w, hist, out)
+    T = proj.shape[0]
+    taps = taps_w.shape[1]
+    _f32("taps_w", taps_w, C * taps); _f32("hist", hist); _f32("out", out, T * C)
+    if proj.stride(1) != 1 or proj.shape[1] < C or (taps > 1 and tuple(hist.shape[1:]) != (taps - 1, C)):
+        raise KernelError("conv_prepare: shapes do not fit")
+    _call("blm_conv_prepare", proj.data_ptr(), _code(proj), proj.stride(0), taps_w.data_ptr(), taps, hist.data_ptr(),
+          out.data_ptr(), step.token_seq.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs,
+          C, G, dk, _stream())
+    return out
+
+
+def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_w, eps, state, out, step, H, G, dk, dv):
+    """The delta rule with a decay per key channel over conv_prepare's rows; see the kernel for the formulas.
+    beta_src: the tensor whose column beta_col + h holds head h's write-strength logit; decay_in [T, H dk] and
+    gate_in [T, H dv] in the same dtype; out [T, H * dv] in that dtype."""
+    _gpu(qkv, beta_src, decay_in, dt_bias, a_log, gate_in, norm_w, state, out)
+    T, C = qkv.shape
+    _f32("qkv", qkv); _f32("dt_bias", dt_bias, H * dk); _f32("a_log", a_log, H); _f32("norm_w", norm_w, dv)
+    _f32("state", state)
+    _contig("decay_in", decay_in); _contig("gate_in", gate_in); _contig("out", out)
+    if not (beta_src.dtype == decay_in.dtype == gate_in.dtype == out.dtype) or beta_src.stride(1) != 1:
+        raise KernelError("delta_scan: the projections and the output must share a dtype")
+    if tuple(decay_in.shape) != (T, H * dk) or tuple(gate_in.shape) != (T, H * dv) or tuple(out.shape) != (T, H * dv) \
+            or tuple(state.shape[1:]) != (H, dk, dv) or beta_col + H > beta_src.shape[1]:
+        raise KernelError("delta_scan: shapes do not fit")
+    _call("blm_delta_scan", qkv.data_ptr(), C, beta_src.data_ptr(), _code(out), beta_src.stride(0), beta_col,
+          decay_in.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(), gate_in.data_ptr(), norm_w.data_ptr(), float(eps),
+          state.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), step.n_seqs, H, G, dk,
+          dv, _stream())
+    return out

@@ -56,7 +56,7 @@ def load_model(folder, dtype="bfloat16", device="cuda:0", cast_32bit=False):
     arch, cfg = read_config(folder)
     rt = Runtime(dtype=dtype, device=device)
     available = safetensors_io.open_folder(folder)
-    plan = arch.plan(cfg, set(available))
+    plan = arch.plan(cfg, {n: tuple(f.shape(n)) for n, f in available.items()})   # names and shapes
     model = Model(plan)
     tensors = loader.load(folder, model.tensor_specs(), dtype, rt.device, plan.ignorable_tensors, available, cast_32bit)
     _notice_wide(tensors, dtype, folder)
@@ -96,7 +96,7 @@ def random_engine(config: dict, seed=0, dtype="bfloat16", max_tokens=8192, max_s
     rt = Runtime(dtype=dtype, device=device)
     made = dict(random_tensors(arch, cfg, seed, std=std, norm_jitter=norm_jitter, dtype=stored_dtype, device=rt.device,
                                quick=quick_weights))
-    plan = arch.plan(cfg, set(made))
+    plan = arch.plan(cfg, {n: tuple(t.shape) for n, t in made.items()})
     model = Model(plan)
     tensors = loader.place(f"the random checkpoint of {arch.name}", made, model.tensor_specs(), dtype, rt.device,
                            plan.ignorable_tensors)

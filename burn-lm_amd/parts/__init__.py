@@ -4,9 +4,15 @@ from .attention import Attention
 from .base import (Block, FeedForward, KVNeed, Mixer, Norm, Part, PartSpec, PositionEncoding, StateNeed,
                    TensorSpec)
 from .block import PreNormBlock
+from .channel_delta import ChannelDelta
+from .dense_xielu import DenseXielu
 from .embedding import Embedding, LMHead
+from .hgrn2 import HGRN2
+from .latent_attention import LatentAttention
+from .norm_layer import LayerNorm
 from .norm_rms import RMSNorm
 from .rope import RotaryEncoding
+from .streams import HyperBlock, HyperConnection, HyperMixerBlock
 from .swiglu import SwiGLU
 
 registry.register_part("mixer", "attention", Attention)
@@ -16,3 +22,11 @@ registry.register_part("position", "rope", RotaryEncoding)
 registry.register_part("block", "pre_norm", PreNormBlock)
 registry.register_part("embedding", "table", Embedding)
 registry.register_part("head", "linear", LMHead)
+registry.register_part("mixer", "latent_attention", LatentAttention)
+registry.register_part("mixer", "hgrn2", HGRN2)
+registry.register_part("mixer", "channel_delta", ChannelDelta)
+registry.register_part("feed_forward", "dense_xielu", DenseXielu)
+registry.register_part("norm", "layernorm", LayerNorm)
+registry.register_part("connection", "hyper", HyperConnection)
+registry.register_part("block", "hyper", HyperBlock)
+registry.register_part("block", "hyper_mixer_only", HyperMixerBlock)

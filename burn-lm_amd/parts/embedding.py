@@ -12,7 +12,8 @@ from .base import Part, TensorSpec
 
 
 class Embedding(Part):
-    """params: vocab, width.  names: weight."""
+    """params: vocab, width, copies (default 1; more: the residual starts as that many equal streams,
+    [tokens, copies, width]).  names: weight."""
     graph_safe = True
 
     def tensor_specs(self):
@@ -25,15 +26,20 @@ class Embedding(Part):
     def step_bytes(self, rows):
         return rows * self.params["width"] * self.table.element_size()      # the rows that are looked up
 
+    def _rows(self, ids):
+        copies = int(self.params.get("copies", 1))
+        shape = (ids.shape[0], self.params["width"]) if copies == 1 else (ids.shape[0], copies, self.params["width"])
+        return torch.empty(shape, dtype=torch.float32, device=ids.device)
+
     def forward(self, ids):
-        h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
+        h = self._rows(ids)
         return self.rt.ops.embed_gather(self.table, ids, h)
 
     def forward_from(self, ids, source_rows, source_cell):
         """The same where some tokens are still on the device: row t is element source_rows[t] of the
         array whose address is in source_cell, where source_rows[t] >= 0.  An embedding without this
         method gets its tokens gathered by a separate launch before the step."""
-        h = torch.empty(ids.shape[0], self.params["width"], dtype=torch.float32, device=ids.device)
+        h = self._rows(ids)
         return self.rt.ops.embed_gather_from(self.table, ids, source_rows, source_cell, h)
 
 

@@ -1,0 +1,56 @@
+"""HGRN2: a gated linear recurrence in which the forget gate also decides what is written.
+
+``q = silu(W_q x)``, ``v = W_v x``, ``f = low + (1 - low) * sigmoid(W_f x + b_f)`` per head and key channel
+(``low`` a stored lower bound); per head ``S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T`` and ``o_t = S_t^T q_t``
+(no key, no other scale); every head's ``o`` is RMS-normed over its value lanes with one shared weight, the heads
+are concatenated and projected.  ``S`` starts at zero, is float32 and is carried per sequence as fixed-size state."""
+from __future__ import annotations
+
+import torch
+
+from .base import Mixer, StateNeed, TensorSpec
+
+
+class HGRN2(Mixer):
+    """params: width, heads, dim, vdim, eps.  names: q, f, f_bias, lower, v, norm, o."""
+    graph_safe = True
+
+    def tensor_specs(self):
+        p, n = self.params, self.names
+        d, H, dk, dv = p["width"], p["heads"], p["dim"], p["vdim"]
+        return {n["q"]: TensorSpec((H * dk, d)), n["f"]: TensorSpec((H * dk, d)), n["f_bias"]: TensorSpec((H * dk,)),
+                n["lower"]: TensorSpec((H * dk,)), n["v"]: TensorSpec((H * dv, d)), n["norm"]: TensorSpec((dv,)),
+                n["o"]: TensorSpec((d, H * dv))}
+
+    def cache_need(self):
+        p = self.params
+        return StateNeed((p["heads"], p["dim"], p["vdim"]), torch.float32)
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        p, n = self.params, self.names
+        self.H, self.dk, self.dv, self.eps = p["heads"], p["dim"], p["vdim"], float(p["eps"])
+        ws = [tensors[n[r]] for r in ("q", "f", "v")]
+        if len({w.dtype for w in ws}) != 1:
+            ws = [w.float() for w in ws]
+        self.w_in = rt.weight(torch.cat(ws, dim=0))
+        self.f_bias = tensors[n["f_bias"]].float().contiguous()
+        self.low = tensors[n["lower"]].float().contiguous()
+        self.norm_w = tensors[n["norm"]].float().contiguous()
+        self.w_o = rt.weight(tensors[n["o"]])
+
+    def step_bytes(self, rows):
+        return sum(w.w.numel() * w.w.element_size() for w in (self.w_in, self.w_o))
+
+    def step_flops(self, rows):
+        return 2 * rows * (self.w_in.w.numel() + self.w_o.w.numel())
+
+    def mixing_flops(self, past, new):
+        return 4 * self.H * self.dk * self.dv * new
+
+    def forward(self, x, step, view):
+        rt = self.rt
+        proj = rt.linear(x, self.w_in)
+        out = torch.zeros(x.shape[0], self.H * self.dv, dtype=rt.dtype, device=x.device)
+        rt.ops.hgrn2_scan(proj, self.f_bias, self.low, self.norm_w, self.eps, view.tensor, out, step, self.H, self.dk, self.dv)
+        return rt.linear(out, self.w_o, partials=True)

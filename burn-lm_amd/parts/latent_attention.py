@@ -1,0 +1,87 @@
+"""Attention whose keys and values are expanded from one low-rank latent per token (latent attention).
+
+``q = W_q x`` per head as ``[dim plain lanes | rot_dim lanes turned by position]``; ``W_dkv x`` gives the latent
+``c`` (kv_rank lanes, RMS-normed with a weight) and one turned key part shared by all heads (rot_dim lanes).
+A head's plain key is ``W_uk c`` and its value ``W_uv c``; score = (q_plain . k_plain + q_rot . k_rot) * scale,
+causal softmax, output projection over the concatenated heads.  Only ``[c | k_rot]`` is cached: the scores are
+computed as ``(W_uk^T q_plain) . c`` and the values applied as ``W_uv (sum_j p_j c_j)``, which is the same
+function, so the cache holds one row of kv_rank + rot_dim lanes per token for all heads and no value pages.
+Rotation: lane i of the first ``rot_dims`` turned lanes pairs with lane i + rot_dims/2."""
+from __future__ import annotations
+
+import torch
+
+from .base import KVNeed, Mixer, TensorSpec
+
+DECODE_BLOCKS_PER_UNIT = 2     # blocks of four (token, head) wavefronts the split decode aims for per compute unit
+
+
+class LatentAttention(Mixer):
+    """params: width, heads, dim, rot_dim, vdim, kv_rank, scale, rot_dims, eps, position (the rotary table's
+    owner, given by the model builder).  names: q, dkv, dkv_norm, uk, uv, o."""
+    graph_safe = True
+
+    def tensor_specs(self):
+        p, n = self.params, self.names
+        d, H, dn, dr, dv, R = p["width"], p["heads"], p["dim"], p["rot_dim"], p["vdim"], p["kv_rank"]
+        return {n["q"]: TensorSpec((H * (dn + dr), d)), n["dkv"]: TensorSpec((R + dr, d)),
+                n["dkv_norm"]: TensorSpec((R,)), n["uk"]: TensorSpec((H * dn, R)), n["uv"]: TensorSpec((H * dv, R)),
+                n["o"]: TensorSpec((d, H * dv))}
+
+    def cache_need(self):
+        p = self.params
+        return KVNeed(1, p["kv_rank"] + p["rot_dim"], 0, no_values=True)
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        p, n = self.params, self.names
+        self.H, self.dn, self.dr, self.dv, self.R = p["heads"], p["dim"], p["rot_dim"], p["vdim"], p["kv_rank"]
+        self.scale, self.eps, self.rot = float(p["scale"]), float(p["eps"]), int(p["rot_dims"])
+        if self.rot % 2 or not 0 <= self.rot <= self.dr:
+            raise ValueError(f"{self.rot} turning lanes do not fit a turned part of {self.dr} lanes")
+        self.position = p["position"]
+        ws = [tensors[n["q"]], tensors[n["dkv"]]]
+        if ws[0].dtype != ws[1].dtype:
+            ws = [w.float() for w in ws]
+        self.n_q = ws[0].shape[0]
+        self.w_in = rt.weight(torch.cat(ws, dim=0))
+        self.norm_w = tensors[n["dkv_norm"]].float().contiguous()
+        H, dn, dv, R = self.H, self.dn, self.dv, self.R
+        self.w_uk_t = tensors[n["uk"]].view(H, dn, R).transpose(1, 2).contiguous()   # [H, R, dn]: q_plain -> latent lanes
+        self.w_uv = tensors[n["uv"]].view(H, dv, R).contiguous()
+        self.w_o = rt.weight(tensors[n["o"]])
+        rt.ops.latent_attn_init(rt.device)
+
+    def step_bytes(self, rows):
+        return sum(w.numel() * w.element_size() for w in (self.w_in.w, self.w_o.w, self.w_uk_t, self.w_uv))
+
+    def step_flops(self, rows):
+        return 2 * rows * (self.w_in.w.numel() + self.w_o.w.numel() + self.w_uk_t.numel() + self.w_uv.numel())
+
+    def mixing_flops(self, past, new):
+        """Scores over kv_rank + rot_dim lanes and weighted latents over kv_rank lanes, per (query, visible row, head)."""
+        pairs = new * past + new * (new + 1) // 2
+        return 2 * self.H * (2 * self.R + self.dr) * pairs
+
+    def forward(self, x, step, view):
+        rt, ops = self.rt, self.rt.ops
+        H, dn, dr, dv, R = self.H, self.dn, self.dr, self.dv, self.R
+        T = x.shape[0]
+        qd = rt.linear(x, self.w_in)                         # [T, H (dn + dr) | R + dr]
+        q, down = qd[:, :self.n_q], qd[:, self.n_q:]
+        qabs = torch.empty(T, H, R + dr, dtype=torch.float32, device=x.device)
+        table = view.block_table(step)
+        ops.latent_write(down, q, self.norm_w, self.eps, self.position.table, self.rot, qabs, view.k, step, table,
+                         view.page_size, H, dn, R, dr, write_kv=view.store)
+        ops.head_project(q, dn + dr, self.w_uk_t, qabs.view(T, H * (R + dr)), R + dr)
+        olat = torch.empty(T, H, R, dtype=torch.float32, device=x.device)
+        n_splits = 1
+        if step.max_new == 1:
+            chunks = (step.max_len_after + 63) // 64
+            blocks = (T * H + 3) // 4
+            n_splits = max(1, min(chunks, (DECODE_BLOCKS_PER_UNIT * rt.compute_units) // blocks,
+                                  ops.latent_attn_max_splits(T, H, R)))
+        ops.latent_attn(qabs, olat, view.k, step, table, view.page_size, H, R, dr, self.scale, n_splits)
+        o = torch.empty(T, H * dv, dtype=rt.dtype, device=x.device)
+        ops.head_project(olat.view(T, H * R), R, self.w_uv, o, dv)
+        return rt.linear(o, self.w_o, partials=True)

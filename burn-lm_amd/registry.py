@@ -34,7 +34,7 @@ class Architecture:
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 _PARTS: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
-                                      "embedding": {}, "head": {}}
+                                      "embedding": {}, "head": {}, "connection": {}}
 
 
 def register_architecture(arch: Architecture, *aliases: str) -> None:
@@ -73,15 +73,17 @@ def parts(family: str) -> Dict[str, type]:
 
 
 def architecture_of(config_dict: dict) -> Architecture:
-    """The architecture a config.json names, by ``architectures[0]`` and then ``model_type``."""
+    """The architecture a config.json names, by ``architectures[0]``, ``architecture`` and then ``model_type``."""
     names = []
     a = config_dict.get("architectures")
     if isinstance(a, list):
         names += [x for x in a if isinstance(x, str)]
+    if isinstance(config_dict.get("architecture"), str):
+        names.append(config_dict["architecture"])
     if isinstance(config_dict.get("model_type"), str):
         names.append(config_dict["model_type"])
     if not names:
-        raise RegistryError("config.json names no architecture (keys 'architectures' or 'model_type'); known: "
+        raise RegistryError("config.json names no architecture (keys 'architectures', 'architecture' or 'model_type'); known: "
                             + ", ".join(sorted(_ARCHITECTURES)))
     for n in names:
         if n in _ARCHITECTURES:

@@ -99,6 +99,14 @@ class Range:
 
 
 @dataclass(frozen=True)
+class Uniform:
+    """Evenly spread over [lo, hi): lo + (hi - lo) * k / 2^24 with k a uniform 24-bit integer."""
+    lo: float
+    hi: float
+    layout: str = "vector"
+
+
+@dataclass(frozen=True)
 class IntegerTable:
     """Integers in [0, n), for tensors kept as int32 (routing tables and the like)."""
     n: int
@@ -143,6 +151,11 @@ def make_tensor(name, shape, init, seed, std=0.02, norm_jitter=0.0, dtype=torch.
             ramp = ramp.reshape(shape[1], shape[0]).t()
         return ramp.reshape(shape).to(dtype).contiguous()
     key = tensor_key(seed, name)
+    if isinstance(init, Uniform):
+        chunk = CHUNK[torch.device(device).type]
+        parts = [uniform_integers(key, a, min(chunk, n - a), 1 << 24, device) for a in range(0, n, chunk)]
+        u = torch.cat(parts).to(torch.float32) * (1.0 / (1 << 24))
+        return (u * float(init.hi - init.lo) + float(init.lo)).to(dtype).reshape(shape)
     if isinstance(init, Ones):
         jitter = norm_jitter if init.jitter is None else init.jitter
         if not jitter:
@@ -152,7 +165,7 @@ def make_tensor(name, shape, init, seed, std=0.02, norm_jitter=0.0, dtype=torch.
         scale, offset = float(std if init.std is None else init.std), 0.0
     else:
         raise ValueError(f"random weights: {name} has the initialiser {init!r}, which is none of "
-                         f"Normal, Ones, Range, IntegerTable or a role name")
+                         f"Normal, Ones, Uniform, Range, IntegerTable or a role name")
     if quick:
         g = torch.Generator(device=device)
         g.manual_seed(tensor_key(seed, name) & 0x7FFFFFFF)
