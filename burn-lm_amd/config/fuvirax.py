@@ -18,6 +18,7 @@ MIXER_KEYS = {
     "channel_delta": dict(conv=int, dim=int, heads=int, kv_heads=int, vdim=int),
 }
 DEFAULT_LOW_RANK = 16
+MAX_POSITIONS = 1 << 20     # the design has no limit of its own; the cache's size decides
 
 
 def _get(d, key, kind, where):
@@ -70,6 +71,10 @@ class FuviraxConfig:
     @property
     def vocab_size(self):
         return self.vocab
+
+    @property
+    def max_positions(self):
+        return MAX_POSITIONS
 
     def order(self):
         """Indices of the layers in the order they run."""

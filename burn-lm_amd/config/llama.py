@@ -81,6 +81,11 @@ class LlamaConfig:
     extra: dict = field(default_factory=dict, compare=False, hash=False)
 
     # -------------------------------------------------------------------------------------
+    @property
+    def max_positions(self):
+        """Longest sequence the model was built for (the name every architecture's configuration answers to)."""
+        return self.max_position_embeddings
+
     @staticmethod
     def from_dict(d: dict) -> "LlamaConfig":
         if not isinstance(d, dict):

@@ -11,13 +11,12 @@ Checkpoint tensor names: ``embed``; per layer i ``l<i>.norm1`` (+ ``.b``), ``l<i
 ``l<i>.shift``, ``l<i>.hc1/2.in|out|mix``, ``l<i>.mix.*``, ``l<i>.mlp.up|down|act``; ``final.norm`` (+ ``.b``)."""
 from __future__ import annotations
 
-from ..config.fuvirax import DEFAULT_LOW_RANK, FuviraxConfig
+from ..config.fuvirax import DEFAULT_LOW_RANK, MAX_POSITIONS, FuviraxConfig
 from ..parts.base import PartSpec
 from ..registry import Architecture, register_architecture
 from ..weights.random_init import Normal, Ones, Uniform
 from .plan import LayerPlan, ModelPlan, Place
 
-MAX_POSITIONS = 1 << 20     # the design has no limit of its own; the cache's size decides
 
 
 def _shape_of(checkpoint, name):

@@ -102,7 +102,7 @@ class InferenceServer:
         from .engine.loading import load_engine, read_config
         t0 = time.perf_counter()
         _, cfg = read_config(self.folder)
-        ctx = min(self.config.max_seq_len, cfg.max_position_embeddings)
+        ctx = min(self.config.max_seq_len, cfg.max_positions)   # every typed configuration says how far its positions go
         self.engine = load_engine(self.folder, dtype=self.dtype, max_tokens=ctx * self.batch_size,
                                   max_seqs=self.batch_size, max_context=ctx, device=self.device,
                                   cast_32bit=self.cast_32bit)
