@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 _lib = None
 _lock = threading.Lock()
 
@@ -39,12 +39,12 @@ _SIGNATURES = {
     "blm_latent_attn": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int,
                         _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_hgrn2_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p,
-                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                       _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_conv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_delta_scan": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                       _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                       _c_int, _c_void_p],
+                       _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_void_p],
     "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p, _c_int,
                         _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -930,18 +930,20 @@ def latent_attn(qabs, olat, kcache, step, block_table, page_size, H, R, Dr, scal
 
 # ------------------------------------------------------------------------------------------
 # recurrent mixers
-def hgrn2_scan(proj, f_bias, low, norm_w, eps, state, out, step, H, dk, dv):
+def hgrn2_scan(proj, f_bias, low, norm_w, eps, state, o_raw, out, step, H, dk, dv):
     """proj [T, >= 2 H dk + H dv]: queries, forget-gate logits, values.  state float32 [slots, H, dk, dv] is read
-    and left updated for the step's sequences; out [T, H * dv] in proj's dtype."""
-    _gpu(proj, f_bias, low, norm_w, state, out)
+    and left updated for the step's sequences; o_raw: zeroed float32 [T, H * dv] for the unnormalised results;
+    out [T, H * dv] in proj's dtype."""
+    _gpu(proj, f_bias, low, norm_w, state, o_raw, out)
+    _f32("o_raw", o_raw, proj.shape[0] * H * dv)
     _f32("f_bias", f_bias, H * dk); _f32("low", low, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
     _contig("out", out)
     if proj.stride(1) != 1 or out.dtype != proj.dtype or tuple(out.shape) != (proj.shape[0], H * dv) \
             or tuple(state.shape[1:]) != (H, dk, dv):
         raise KernelError("hgrn2_scan: shapes do not fit")
     _call("blm_hgrn2_scan", proj.data_ptr(), _code(proj), proj.stride(0), f_bias.data_ptr(), low.data_ptr(),
-          norm_w.data_ptr(), float(eps), state.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
-          step.seq_slots.data_ptr(), step.n_seqs, H, dk, dv, _stream())
+          norm_w.data_ptr(), float(eps), state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
+          step.seq_slots.data_ptr(), proj.shape[0], step.n_seqs, H, dk, dv, _stream())
     return out
 
 
@@ -961,12 +963,14 @@ def conv_prepare(proj, taps_w, hist, out, step, C, G, dk):
     return out
 
 
-def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_w, eps, state, out, step, H, G, dk, dv):
+def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_w, eps, state, o_raw, out, step, H, G,
+               dk, dv):
     """The delta rule with a decay per key channel over conv_prepare's rows; see the kernel for the formulas.
     beta_src: the tensor whose column beta_col + h holds head h's write-strength logit; decay_in [T, H dk] and
-    gate_in [T, H dv] in the same dtype; out [T, H * dv] in that dtype."""
-    _gpu(qkv, beta_src, decay_in, dt_bias, a_log, gate_in, norm_w, state, out)
+    gate_in [T, H dv] in the same dtype; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in that dtype."""
+    _gpu(qkv, beta_src, decay_in, dt_bias, a_log, gate_in, norm_w, state, o_raw, out)
     T, C = qkv.shape
+    _f32("o_raw", o_raw, T * H * dv)
     _f32("qkv", qkv); _f32("dt_bias", dt_bias, H * dk); _f32("a_log", a_log, H); _f32("norm_w", norm_w, dv)
     _f32("state", state)
     _contig("decay_in", decay_in); _contig("gate_in", gate_in); _contig("out", out)
@@ -977,6 +981,6 @@ def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_
         raise KernelError("delta_scan: shapes do not fit")
     _call("blm_delta_scan", qkv.data_ptr(), C, beta_src.data_ptr(), _code(out), beta_src.stride(0), beta_col,
           decay_in.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(), gate_in.data_ptr(), norm_w.data_ptr(), float(eps),
-          state.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), step.n_seqs, H, G, dk,
-          dv, _stream())
+          state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T,
+          step.n_seqs, H, G, dk, dv, _stream())
     return out

@@ -1,11 +1,13 @@
 // Recurrent mixers whose state is a matrix [key channels][value channels] per head and sequence, kept in
 // float in the cache's state tensors: a gated linear recurrence whose forget gate also weighs the write
-// (HGRN2), and a delta rule with one decay per key channel.  One block per (sequence, head) walks the
-// sequence's tokens of the step in order; thread j owns column j of the state (all key channels of one
-// value channel) in registers, so a token costs each thread two passes over its column and the block one
-// reduction for the norm of the head's result.  Columns are independent of each other; what a token needs
-// of the key side (gates, keys, queries: one value per key channel) is prepared by the block's threads
-// together in shared memory.  The same kernels serve prompts and decoding (a sequence then brings one token).
+// (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
+// channel) never meet: each needs only its own value and what the token brings per key channel (gates, keys,
+// queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns: lane (g, c) keeps rows
+// g, g + 4, g + 8, ... of column c in registers, the four lanes of a column add their parts of a dot product
+// with two cross-lane steps, and nothing waits for another wavefront.  What a token brings per key channel is
+// computed by the wavefront into its own piece of shared memory, from inputs it loaded one token ahead.  The
+// results go out unnormalised in float; a second kernel takes the root mean square over each head's value
+// lanes, the weight and (delta rule) the output gate.  The same kernels serve prompts and decoding.
 //
 // Also here: the short causal convolution in front of the delta rule with its per-sequence history.
 #include "common.h"
@@ -14,88 +16,167 @@ __device__ __forceinline__ float blm_sigmoid(float z) { return 1.0f / (1.0f + ex
 __device__ __forceinline__ float blm_silu(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float blm_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
+#define SCAN_COLS 16      // columns of the state per wavefront
+#define SCAN_GROUPS 4     // lanes per column; lane (g, c) holds rows g, g + 4, ...
+#define SCAN_WAVES 4
+#define SCAN_MAX_DK 256
+
 // ---------------------------------------------------------------------------------------
 // HGRN2.  proj [T][ld]: q at column 0 (H*dk), forget-gate logits at H*dk (H*dk), values at 2*H*dk (H*dv).
 //   f = low + (1 - low) * sigmoid(logit + bias);  S = diag(f) S + (1 - f) v^T;  o = S^T silu(q)
-//   out = o / sqrt(mean(o^2) + eps) * norm_w      (per head, over its dv lanes)
-// state [slots][H][dk][dv] float.
+// state [slots][H][dk][dv] float; o_raw [T][H*dv] float.
 // ---------------------------------------------------------------------------------------
-template <typename TA, int DK>
-__global__ void hgrn2_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ f_bias,
-                                  const float* __restrict__ low, const float* __restrict__ norm_w, float eps,
-                                  float* __restrict__ state, TA* __restrict__ out, const int* __restrict__ cu_seqlens,
-                                  const int* __restrict__ seq_slots, int H, int dk, int dv) {
-  extern __shared__ float sm[];          // two buffers of [f (dk) | q (dk)]
-  __shared__ float red[17];
-  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+template <typename TA, int ROWS>
+__global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
+    hgrn2_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ f_bias,
+                      const float* __restrict__ low, float* __restrict__ state, float* __restrict__ o_raw,
+                      const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv,
+                      int col_groups, long long n_items) {
+  __shared__ float sm[SCAN_WAVES][2][2 * SCAN_MAX_DK];     // per wavefront, two tokens: [f | q]
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
+  if (item >= n_items) return;
+  const int cg = (int)(item % col_groups);
+  const int h = (int)((item / col_groups) % H);
+  const int b = (int)(item / ((long long)col_groups * H));
   const int slot = seq_slots[b];
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
   if (slot < 0 || t1 <= t0) return;
+  const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
+  const bool own = col < dv;
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
-  float S[DK];
-  const bool own = j < dv;
+  float S[ROWS];
 #pragma unroll
-  for (int i = 0; i < DK; ++i) S[i] = (own && i < dk) ? S_g[(size_t)i * dv + j] : 0.f;
-  const float nw = own ? norm_w[j] : 0.f;
-  for (int t = t0; t < t1; ++t) {
-    float* fq = sm + (size_t)((t - t0) & 1) * 2 * dk;
+  for (int r = 0; r < ROWS; ++r) {
+    const int i = r * SCAN_GROUPS + g;
+    S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
+  }
+  // per key channel (lane l computes channels l, l + 64, ...): constants, and the token's raw inputs one ahead
+  constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
+  float lo[PER], fb[PER], raw_f[PER], raw_q[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = lane + k * BLM_WAVE;
+    lo[k] = i < dk ? low[h * dk + i] : 0.f;
+    fb[k] = i < dk ? f_bias[h * dk + i] : 0.f;
+  }
+  auto load_raw = [&](int t, float& v) {
     const TA* row = proj + (size_t)t * ld;
-    for (int i = j; i < dk; i += blockDim.x) {
-      const float lo = low[h * dk + i];
-      fq[i] = lo + (1.f - lo) * blm_sigmoid(to_float(row[(size_t)H * dk + h * dk + i]) + f_bias[h * dk + i]);
-      fq[dk + i] = blm_silu(to_float(row[h * dk + i]));
-    }
-    const float v = own ? to_float(row[(size_t)2 * H * dk + h * dv + j]) : 0.f;
-    __syncthreads();
-    float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < DK; ++i) {
+    for (int k = 0; k < PER; ++k) {
+      const int i = lane + k * BLM_WAVE;
       if (i < dk) {
-        const float f = fq[i];
-        S[i] = fmaf(f, S[i], (1.f - f) * v);
-        o = fmaf(S[i], fq[dk + i], o);
+        raw_f[k] = to_float(row[(size_t)H * dk + h * dk + i]);
+        raw_q[k] = to_float(row[h * dk + i]);
       }
     }
-    const float ss = block_sum(own ? o * o : 0.f, red);
-    if (own) out[(size_t)t * H * dv + h * dv + j] = from_float<TA>(o * (1.0f / sqrtf(ss / (float)dv + eps)) * nw);
+    v = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
+  };
+  float v_next;
+  load_raw(t0, v_next);
+  for (int t = t0; t < t1; ++t) {
+    float* fq = sm[wave][(t - t0) & 1];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int i = lane + k * BLM_WAVE;
+      if (i < dk) {
+        fq[i] = lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[k] + fb[k]);
+        fq[dk + i] = blm_silu(raw_q[k]);
+      }
+    }
+    const float v = v_next;
+    if (t + 1 < t1) load_raw(t + 1, v_next);
+    __builtin_amdgcn_wave_barrier();      // the piece of shared memory is the wavefront's own: reads follow writes in order
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = r * SCAN_GROUPS + g;
+      if (i < dk) {
+        const float f = fq[i];
+        S[r] = fmaf(f, S[r], (1.f - f) * v);
+        o = fmaf(S[r], fq[dk + i], o);
+      }
+    }
+    o = rows_sum(o);
+    if (own && g == 0) o_raw[(size_t)t * H * dv + h * dv + col] = o;
+    __builtin_amdgcn_wave_barrier();
   }
   if (own) {
 #pragma unroll
-    for (int i = 0; i < DK; ++i)
-      if (i < dk) S_g[(size_t)i * dv + j] = S[i];
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = r * SCAN_GROUPS + g;
+      if (i < dk) S_g[(size_t)i * dv + col] = S[r];
+    }
   }
 }
 
-#define BLM_SCAN_PICK(CALL)                  \
-  do {                                       \
-    if (dk <= 16) { CALL(16); }              \
-    else if (dk <= 32) { CALL(32); }         \
-    else if (dk <= 64) { CALL(64); }         \
-    else if (dk <= 128) { CALL(128); }       \
-    else { CALL(256); }                      \
+// out[t][h][j] = o_raw[t][h][j] / sqrt(mean_j(o_raw^2) + eps) * norm_w[j] (* sigmoid(gate[t][h][j])); one wavefront
+// per (token, head).  Rows of padding tokens hold whatever o_raw holds (the caller clears it).
+template <typename TA>
+__global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
+    head_norm_kernel(const float* __restrict__ o_raw, const float* __restrict__ norm_w, const TA* __restrict__ gate,
+                     TA* __restrict__ out, long long n_items, int dv, float eps) {
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
+  if (item >= n_items) return;
+  const float* src = o_raw + (size_t)item * dv;
+  float ss = 0.f;
+  for (int j = lane; j < dv; j += BLM_WAVE) ss = fmaf(src[j], src[j], ss);
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+  for (int j = lane; j < dv; j += BLM_WAVE) {
+    float v = src[j] * inv * norm_w[j];
+    if (gate) v *= blm_sigmoid(to_float(gate[(size_t)item * dv + j]));
+    out[(size_t)item * dv + j] = from_float<TA>(v);
+  }
+}
+
+static int launch_head_norm(const float* o_raw, const float* norm_w, const void* gate, void* out, int dtype, long long items,
+                            int dv, float eps, hipStream_t stream) {
+  const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(head_norm_kernel<float>, dim3(blocks), dim3(SCAN_WAVES * BLM_WAVE), 0, stream, o_raw, norm_w,
+                       (const float*)gate, (float*)out, items, dv, eps);
+  else
+    hipLaunchKernelGGL(head_norm_kernel<bf16>, dim3(blocks), dim3(SCAN_WAVES * BLM_WAVE), 0, stream, o_raw, norm_w,
+                       (const bf16*)gate, (bf16*)out, items, dv, eps);
+  BLM_LAUNCH_CHECK("head_norm");
+  return 0;
+}
+
+// rows per lane: the key channels dealt to four lanes, rounded up to what the kernels are built for
+#define BLM_SCAN_PICK(CALL)                   \
+  do {                                        \
+    const int rows = (dk + 3) / 4;            \
+    if (rows <= 4) { CALL(4); }               \
+    else if (rows <= 8) { CALL(8); }          \
+    else if (rows <= 16) { CALL(16); }        \
+    else if (rows <= 32) { CALL(32); }        \
+    else { CALL(64); }                        \
   } while (0)
 
 extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* f_bias, const float* low,
-                              const float* norm_w, float eps, float* state, void* out, const int* cu_seqlens,
-                              const int* seq_slots, int B, int H, int dk, int dv, hipStream_t stream) {
-  BLM_REQUIRE(B > 0 && H > 0 && H <= 65535, "hgrn2_scan: bad sizes B=%d H=%d", B, H);
-  BLM_REQUIRE(dk >= 1 && dk <= 256 && dv >= 1 && dv <= 1024, "hgrn2_scan: a head of %d x %d is not supported (up to 256 x 1024)", dk, dv);
+                              const float* norm_w, float eps, float* state, float* o_raw, void* out,
+                              const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv,
+                              hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && B > 0 && H > 0, "hgrn2_scan: bad sizes T=%d B=%d H=%d", T, B, H);
+  BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "hgrn2_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(ld >= 2 * H * dk + H * dv, "hgrn2_scan: rows of %d are too short", ld);
-  const int threads = (dv + BLM_WAVE - 1) / BLM_WAVE * BLM_WAVE;
-  const size_t smem = (size_t)4 * dk * sizeof(float);
-  dim3 grid(B, H), block(threads);
-#define BLM_HG(DK)                                                                                                       \
-  if (dtype == BLM_F32)                                                                                                  \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<float, DK>), grid, block, smem, stream, (const float*)proj, ld, f_bias, low,   \
-                       norm_w, eps, state, (float*)out, cu_seqlens, seq_slots, H, dk, dv);                               \
-  else                                                                                                                   \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, DK>), grid, block, smem, stream, (const bf16*)proj, ld, f_bias, low,     \
-                       norm_w, eps, state, (bf16*)out, cu_seqlens, seq_slots, H, dk, dv)
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "hgrn2_scan: unsupported dtype %d", dtype);
+  const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
+  const long long items = (long long)B * H * col_groups;
+  const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
+  dim3 grid(blocks), block(SCAN_WAVES * BLM_WAVE);
+#define BLM_HG(ROWS)                                                                                                   \
+  if (dtype == BLM_F32)                                                                                                \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), grid, block, 0, stream, (const float*)proj, ld, f_bias, low,  \
+                       state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                             \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), grid, block, 0, stream, (const bf16*)proj, ld, f_bias, low,    \
+                       state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_HG);
 #undef BLM_HG
   BLM_LAUNCH_CHECK("hgrn2_scan");
-  return 0;
+  return launch_head_norm(o_raw, norm_w, nullptr, out, dtype, (long long)T * H, dv, eps, stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -203,92 +284,129 @@ extern "C" int blm_conv_prepare(const void* proj, int dtype, int ld, const float
 // head h reads q/k head h / (H / G)).  beta = sigmoid(beta_logit[t][h]); decay_i = exp(-exp(a_log[h]) *
 // softplus(decay_in[t][h*dk+i] + dt_bias[h*dk+i])); per token, in this order:
 //   S = diag(decay) S;  u = beta (v - S^T k);  S = S + k u^T;  o = S^T q
-//   out = o / sqrt(mean(o^2) + eps) * norm_w * sigmoid(gate_in[t][h*dv+j])
+// then out = o / sqrt(mean(o^2) + eps) * norm_w * sigmoid(gate_in[t][h*dv+j]) by head_norm_kernel.
 // beta_logit: column `beta_col` of rows of `ld_beta` elements; decay_in, gate_in: [T][H*dk], [T][H*dv].
 // ---------------------------------------------------------------------------------------
-template <typename TA, int DK>
-__global__ void delta_scan_kernel(const float* __restrict__ qkv, int C, const TA* __restrict__ beta_src, int ld_beta,
-                                  int beta_col, const TA* __restrict__ decay_in, const float* __restrict__ dt_bias,
-                                  const float* __restrict__ a_log, const TA* __restrict__ gate_in,
-                                  const float* __restrict__ norm_w, float eps, float* __restrict__ state,
-                                  TA* __restrict__ out, const int* __restrict__ cu_seqlens,
-                                  const int* __restrict__ seq_slots, int H, int G, int dk, int dv) {
-  extern __shared__ float sm[];          // two buffers of [decay (dk) | k (dk) | q (dk) | beta (1)]
-  __shared__ float red[17];
-  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+template <typename TA, int ROWS>
+__global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
+    delta_scan_kernel(const float* __restrict__ qkv, int C, const TA* __restrict__ beta_src, int ld_beta, int beta_col,
+                      const TA* __restrict__ decay_in, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                      float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
+                      const int* __restrict__ seq_slots, int H, int G, int dk, int dv, int col_groups, long long n_items) {
+  __shared__ float sm[SCAN_WAVES][2][3 * SCAN_MAX_DK];     // per wavefront, two tokens: [decay | k | q]
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
+  if (item >= n_items) return;
+  const int cg = (int)(item % col_groups);
+  const int h = (int)((item / col_groups) % H);
+  const int b = (int)(item / ((long long)col_groups * H));
   const int slot = seq_slots[b];
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
   if (slot < 0 || t1 <= t0) return;
-  const int g = h / (H / G);
+  const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
+  const bool own = col < dv;
+  const int kh = h / (H / G);
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
-  float S[DK];
-  const bool own = j < dv;
+  float S[ROWS];
 #pragma unroll
-  for (int i = 0; i < DK; ++i) S[i] = (own && i < dk) ? S_g[(size_t)i * dv + j] : 0.f;
-  const float nw = own ? norm_w[j] : 0.f;
+  for (int r = 0; r < ROWS; ++r) {
+    const int i = r * SCAN_GROUPS + g;
+    S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
+  }
+  constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
   const float rate = expf(a_log[h]);
-  const int stride = 3 * dk + 1;
-  for (int t = t0; t < t1; ++t) {
-    float* buf = sm + (size_t)((t - t0) & 1) * stride;
+  float bias[PER], raw_d[PER], raw_k[PER], raw_q[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = lane + k * BLM_WAVE;
+    bias[k] = i < dk ? dt_bias[h * dk + i] : 0.f;
+  }
+  auto load_raw = [&](int t, float& v, float& beta_logit) {
     const float* row = qkv + (size_t)t * C;
-    for (int i = j; i < dk; i += blockDim.x) {
-      buf[i] = expf(-rate * blm_softplus(to_float(decay_in[(size_t)t * H * dk + h * dk + i]) + dt_bias[h * dk + i]));
-      buf[dk + i] = row[(size_t)G * dk + g * dk + i];
-      buf[2 * dk + i] = row[g * dk + i];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int i = lane + k * BLM_WAVE;
+      if (i < dk) {
+        raw_d[k] = to_float(decay_in[(size_t)t * H * dk + h * dk + i]);
+        raw_k[k] = row[(size_t)G * dk + kh * dk + i];
+        raw_q[k] = row[kh * dk + i];
+      }
     }
-    if (j == 0) buf[3 * dk] = blm_sigmoid(to_float(beta_src[(size_t)t * ld_beta + beta_col + h]));
-    const float v = own ? row[(size_t)2 * G * dk + h * dv + j] : 0.f;
-    const float gate = own ? blm_sigmoid(to_float(gate_in[(size_t)t * H * dv + h * dv + j])) : 0.f;
-    __syncthreads();
+    v = own ? row[(size_t)2 * G * dk + h * dv + col] : 0.f;
+    beta_logit = to_float(beta_src[(size_t)t * ld_beta + beta_col + h]);
+  };
+  float v_next, bl_next;
+  load_raw(t0, v_next, bl_next);
+  for (int t = t0; t < t1; ++t) {
+    float* buf = sm[wave][(t - t0) & 1];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int i = lane + k * BLM_WAVE;
+      if (i < dk) {
+        buf[i] = expf(-rate * blm_softplus(raw_d[k] + bias[k]));
+        buf[dk + i] = raw_k[k];
+        buf[2 * dk + i] = raw_q[k];
+      }
+    }
+    const float v = v_next, beta = blm_sigmoid(bl_next);
+    if (t + 1 < t1) load_raw(t + 1, v_next, bl_next);
+    __builtin_amdgcn_wave_barrier();
     float dot = 0.f;
 #pragma unroll
-    for (int i = 0; i < DK; ++i) {
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = r * SCAN_GROUPS + g;
       if (i < dk) {
-        S[i] *= buf[i];
-        dot = fmaf(S[i], buf[dk + i], dot);
+        S[r] *= buf[i];
+        dot = fmaf(S[r], buf[dk + i], dot);
       }
     }
-    const float u = buf[3 * dk] * (v - dot);
+    const float u = beta * (v - rows_sum(dot));
     float o = 0.f;
 #pragma unroll
-    for (int i = 0; i < DK; ++i) {
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = r * SCAN_GROUPS + g;
       if (i < dk) {
-        S[i] = fmaf(buf[dk + i], u, S[i]);
-        o = fmaf(S[i], buf[2 * dk + i], o);
+        S[r] = fmaf(buf[dk + i], u, S[r]);
+        o = fmaf(S[r], buf[2 * dk + i], o);
       }
     }
-    const float ss = block_sum(own ? o * o : 0.f, red);
-    if (own) out[(size_t)t * H * dv + h * dv + j] = from_float<TA>(o * (1.0f / sqrtf(ss / (float)dv + eps)) * nw * gate);
+    o = rows_sum(o);
+    if (own && g == 0) o_raw[(size_t)t * H * dv + h * dv + col] = o;
+    __builtin_amdgcn_wave_barrier();
   }
   if (own) {
 #pragma unroll
-    for (int i = 0; i < DK; ++i)
-      if (i < dk) S_g[(size_t)i * dv + j] = S[i];
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = r * SCAN_GROUPS + g;
+      if (i < dk) S_g[(size_t)i * dv + col] = S[r];
+    }
   }
 }
 
 extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int dtype, int ld_beta, int beta_col,
                               const void* decay_in, const float* dt_bias, const float* a_log, const void* gate_in,
-                              const float* norm_w, float eps, float* state, void* out, const int* cu_seqlens,
-                              const int* seq_slots, int B, int H, int G, int dk, int dv, hipStream_t stream) {
-  BLM_REQUIRE(B > 0 && H > 0 && H <= 65535 && G > 0 && H % G == 0, "delta_scan: bad sizes B=%d H=%d G=%d", B, H, G);
-  BLM_REQUIRE(dk >= 1 && dk <= 256 && dv >= 1 && dv <= 1024, "delta_scan: a head of %d x %d is not supported (up to 256 x 1024)", dk, dv);
+                              const float* norm_w, float eps, float* state, float* o_raw, void* out,
+                              const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int G, int dk, int dv,
+                              hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && B > 0 && H > 0 && G > 0 && H % G == 0, "delta_scan: bad sizes T=%d B=%d H=%d G=%d", T, B, H, G);
+  BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "delta_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(C >= 2 * G * dk + H * dv, "delta_scan: rows of %d are too short", C);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "delta_scan: unsupported dtype %d", dtype);
-  const int threads = (dv + BLM_WAVE - 1) / BLM_WAVE * BLM_WAVE;
-  const size_t smem = (size_t)2 * (3 * dk + 1) * sizeof(float);
-  dim3 grid(B, H), block(threads);
-#define BLM_DS(DK)                                                                                                        \
+  const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
+  const long long items = (long long)B * H * col_groups;
+  const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
+  dim3 grid(blocks), block(SCAN_WAVES * BLM_WAVE);
+#define BLM_DS(ROWS)                                                                                                      \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((delta_scan_kernel<float, DK>), grid, block, smem, stream, qkv, C, (const float*)beta_src, ld_beta, \
-                       beta_col, (const float*)decay_in, dt_bias, a_log, (const float*)gate_in, norm_w, eps, state,       \
-                       (float*)out, cu_seqlens, seq_slots, H, G, dk, dv);                                                 \
+    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), grid, block, 0, stream, qkv, C, (const float*)beta_src, ld_beta, \
+                       beta_col, (const float*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,   \
+                       dv, col_groups, items);                                                                            \
   else                                                                                                                    \
-    hipLaunchKernelGGL((delta_scan_kernel<bf16, DK>), grid, block, smem, stream, qkv, C, (const bf16*)beta_src, ld_beta,   \
-                       beta_col, (const bf16*)decay_in, dt_bias, a_log, (const bf16*)gate_in, norm_w, eps, state,         \
-                       (bf16*)out, cu_seqlens, seq_slots, H, G, dk, dv)
+    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), grid, block, 0, stream, qkv, C, (const bf16*)beta_src, ld_beta,   \
+                       beta_col, (const bf16*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,    \
+                       dv, col_groups, items)
   BLM_SCAN_PICK(BLM_DS);
 #undef BLM_DS
   BLM_LAUNCH_CHECK("delta_scan");
-  return 0;
+  return launch_head_norm(o_raw, norm_w, gate_in, out, dtype, (long long)T * H, dv, eps, stream);
 }

@@ -175,7 +175,7 @@ extern "C" int blm_token_shift(const float* n, const float* mu, const float* sta
 // xIELU: z > 0: a_pos z^2 + z / 2;  z <= 0: a_neg (exp(z) - 1 - z) + z / 2
 // ---------------------------------------------------------------------------------------
 template <typename TA>
-__global__ void xielu_kernel(const TA* __restrict__ in, TA* __restrict__ out, long long n, float a_pos, float a_neg) {
+__global__ void xielu_kernel(const TA* in, TA* out, long long n, float a_pos, float a_neg) {   // out may be in
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     const float z = to_float(in[i]);

@@ -77,15 +77,30 @@ class ChannelDelta(Mixer):
         return t if t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 else t.contiguous()
 
     def forward(self, x, step, view):
-        rt, ops = self.rt, self.rt.ops
-        state, hist = (view[0].tensor, view[1].tensor) if isinstance(view, tuple) else (view.tensor, self.no_hist)
-        T, C = x.shape[0], self.C
+        return self.output(self.scan(self.project(x, step, view), step, view))
+
+    def project(self, x, step, view):
+        """The stacked projection, the convolutions with their activations and unit norms (which also move the
+        sequences' convolution history on), and the two low-rank projections' second halves."""
+        rt, C = self.rt, self.C
+        hist = view[1].tensor if isinstance(view, tuple) else self.no_hist
         proj = rt.linear(x, self.w_in)           # [T, q | k | v | a1 | g1 | b | padding]
-        qkv = torch.empty(T, C, dtype=torch.float32, device=x.device)
-        ops.conv_prepare(proj, self.taps_w, hist, qkv, step, C, self.G, self.dk)
+        qkv = torch.empty(x.shape[0], C, dtype=torch.float32, device=x.device)
+        rt.ops.conv_prepare(proj, self.taps_w, hist, qkv, step, C, self.G, self.dk)
         decay_in = rt.linear(self._aligned(proj[:, C:C + self.ra]), self.w_a2)
         gate_in = rt.linear(self._aligned(proj[:, C + self.ra:C + self.ra + self.rg]), self.w_g2)
-        out = torch.zeros(T, self.H * self.dv, dtype=rt.dtype, device=x.device)
-        ops.delta_scan(qkv, proj, C + self.ra + self.rg, decay_in, self.dt_bias, self.a_log, gate_in, self.norm_w,
-                       self.eps, state, out, step, self.H, self.G, self.dk, self.dv)
-        return rt.linear(out, self.w_o, partials=True)
+        return proj, qkv, decay_in, gate_in
+
+    def scan(self, projected, step, view):
+        """The recurrence over the step's tokens, each sequence from its own state -> [tokens, heads * vdim]."""
+        rt = self.rt
+        proj, qkv, decay_in, gate_in = projected
+        state = view[0].tensor if isinstance(view, tuple) else view.tensor
+        T = qkv.shape[0]
+        o_raw = torch.zeros(T, self.H * self.dv, dtype=torch.float32, device=qkv.device)
+        out = torch.empty(T, self.H * self.dv, dtype=rt.dtype, device=qkv.device)
+        return rt.ops.delta_scan(qkv, proj, self.C + self.ra + self.rg, decay_in, self.dt_bias, self.a_log, gate_in,
+                                 self.norm_w, self.eps, state, o_raw, out, step, self.H, self.G, self.dk, self.dv)
+
+    def output(self, mixed):
+        return self.rt.linear(mixed, self.w_o, partials=True)

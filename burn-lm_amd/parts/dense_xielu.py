@@ -39,4 +39,4 @@ class DenseXielu(FeedForward):
     def forward(self, x, step):
         rt = self.rt
         z = rt.linear(x, self.w_up)
-        return rt.linear(rt.ops.xielu(z, torch.empty_like(z), self.a_pos, self.a_neg), self.w_down, partials=True)
+        return rt.linear(rt.ops.xielu(z, z, self.a_pos, self.a_neg), self.w_down, partials=True)     # in place

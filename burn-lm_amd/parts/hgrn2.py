@@ -49,8 +49,18 @@ class HGRN2(Mixer):
         return 4 * self.H * self.dk * self.dv * new
 
     def forward(self, x, step, view):
+        return self.output(self.scan(self.project(x), step, view))
+
+    def project(self, x):
+        return self.rt.linear(x, self.w_in)
+
+    def output(self, mixed):
+        return self.rt.linear(mixed, self.w_o, partials=True)
+
+    def scan(self, proj, step, view):
+        """The recurrence over the step's tokens, each sequence from its own state -> [tokens, heads * vdim]."""
         rt = self.rt
-        proj = rt.linear(x, self.w_in)
-        out = torch.zeros(x.shape[0], self.H * self.dv, dtype=rt.dtype, device=x.device)
-        rt.ops.hgrn2_scan(proj, self.f_bias, self.low, self.norm_w, self.eps, view.tensor, out, step, self.H, self.dk, self.dv)
-        return rt.linear(out, self.w_o, partials=True)
+        o_raw = torch.zeros(proj.shape[0], self.H * self.dv, dtype=torch.float32, device=proj.device)
+        out = torch.empty(proj.shape[0], self.H * self.dv, dtype=rt.dtype, device=proj.device)
+        return rt.ops.hgrn2_scan(proj, self.f_bias, self.low, self.norm_w, self.eps, view.tensor, o_raw, out, step,
+                                 self.H, self.dk, self.dv)

@@ -64,24 +64,40 @@ class LatentAttention(Mixer):
         return 2 * self.H * (2 * self.R + self.dr) * pairs
 
     def forward(self, x, step, view):
+        return self.output(self.attend(self.project(x, step, view), step, view))
+
+    def project(self, x, step, view):
+        """The absorbed queries [tokens, heads, kv_rank + rot_dim] (float32) of the step's tokens; their latents and
+        turned key parts are in the cache afterwards."""
         rt, ops = self.rt, self.rt.ops
-        H, dn, dr, dv, R = self.H, self.dn, self.dr, self.dv, self.R
+        H, dn, dr, R = self.H, self.dn, self.dr, self.R
         T = x.shape[0]
         qd = rt.linear(x, self.w_in)                         # [T, H (dn + dr) | R + dr]
         q, down = qd[:, :self.n_q], qd[:, self.n_q:]
         qabs = torch.empty(T, H, R + dr, dtype=torch.float32, device=x.device)
-        table = view.block_table(step)
-        ops.latent_write(down, q, self.norm_w, self.eps, self.position.table, self.rot, qabs, view.k, step, table,
-                         view.page_size, H, dn, R, dr, write_kv=view.store)
+        ops.latent_write(down, q, self.norm_w, self.eps, self.position.table, self.rot, qabs, view.k, step,
+                         view.block_table(step), view.page_size, H, dn, R, dr, write_kv=view.store)
         ops.head_project(q, dn + dr, self.w_uk_t, qabs.view(T, H * (R + dr)), R + dr)
-        olat = torch.empty(T, H, R, dtype=torch.float32, device=x.device)
+        return qabs
+
+    def attend(self, qabs, step, view):
+        """Every (token, head)'s weighted sum of the latents it sees -> float32 [tokens, heads, kv_rank]."""
+        rt, ops = self.rt, self.rt.ops
+        H, dr, R = self.H, self.dr, self.R
+        T = qabs.shape[0]
+        olat = torch.empty(T, H, R, dtype=torch.float32, device=qabs.device)
         n_splits = 1
         if step.max_new == 1:
             chunks = (step.max_len_after + 63) // 64
             blocks = (T * H + 3) // 4
             n_splits = max(1, min(chunks, (DECODE_BLOCKS_PER_UNIT * rt.compute_units) // blocks,
                                   ops.latent_attn_max_splits(T, H, R)))
-        ops.latent_attn(qabs, olat, view.k, step, table, view.page_size, H, R, dr, self.scale, n_splits)
-        o = torch.empty(T, H * dv, dtype=rt.dtype, device=x.device)
-        ops.head_project(olat.view(T, H * R), R, self.w_uv, o, dv)
+        return ops.latent_attn(qabs, olat, view.k, step, view.block_table(step), view.page_size, H, R, dr, self.scale,
+                               n_splits)
+
+    def output(self, olat):
+        rt = self.rt
+        T = olat.shape[0]
+        o = torch.empty(T, self.H * self.dv, dtype=rt.dtype, device=olat.device)
+        rt.ops.head_project(olat.view(T, self.H * self.R), self.R, self.w_uv, o, self.dv)
         return rt.linear(o, self.w_o, partials=True)
