@@ -300,6 +300,135 @@ def kernel_rates(engine, batch, context, prefill_tokens):
     return out
 
 
+DESIGN_SIZES = {
+    # layer sizes that resemble a 1B and a 3B model; the Llama beside each has the same width, the same number
+    # of layers and as many feed-forward weights per layer (two matrices of 1.5 x the inner size against three)
+    "1b-like": dict(width=2048, ff=12288, heads=16, llama="llama3.2-1b"),
+    "3b-like": dict(width=3072, ff=12288, heads=24, llama="llama3.2-3b"),
+}
+
+
+def fuvirax_config(width, ff, heads, layers, vocab):
+    """Latent attention, HGRN2 and the delta rule in turn, heads of 128 lanes, a latent of 512 + 64 lanes."""
+    mlp = dict(kind="dense", ff=ff)
+    kinds = [dict(type="latent_attention", mlp=mlp,
+                  mixer=dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, rot=dict(base=500000.0, dims=64),
+                             scale=192 ** -0.5)),
+             dict(type="hgrn2", mlp=mlp, mixer=dict(heads=heads, dim=128, vdim=128)),
+             dict(type="channel_delta", mlp=mlp, mixer=dict(heads=heads, kv_heads=heads // 2, dim=128, vdim=128, conv=4,
+                                                            decay_rank=64, gate_rank=64))]
+    return dict(architecture="Fuvirax", vocab=vocab, width=width, streams=4, logit_scale=1.0, norm=dict(eps=1e-6),
+                layers=[kinds[i % 3] for i in range(layers)])
+
+
+def mixer_rates(engine, batch, context, prefill_tokens):
+    """The mixing kernels of every kind of mixer in the engine alone (no projections), at a decode step of `batch`
+    sequences that hold `context` tokens and at a prompt of `prefill_tokens`: time, and the rate against the limit
+    that binds: decode: bytes of cache rows or state (read and written once) a second; prompts: operations a second."""
+    import torch
+    rt, model = engine.rt, engine.model
+    out, seen = {}, {}
+    for i, pl in enumerate(model.plan.order):
+        m = model.blocks[pl.layer].mixer
+        seen.setdefault(type(m).__name__, (model.blocks[pl.layer], engine.cache.views[i]))
+    width = model.plan.width
+
+    def mixer_view(block, view):
+        return block._views(view)[1] if hasattr(block, "_views") else view
+
+    def run(kind, block, view, step, x, tag, nbytes=None, flops=None):
+        m, v = block.mixer, mixer_view(block, view)
+        if kind == "Attention":
+            mid, mix = m.project(x, step, v), m.attend
+        elif kind == "LatentAttention":
+            mid, mix = m.project(x, step, v), m.attend
+        elif kind == "HGRN2":
+            mid, mix = m.project(x), m.scan
+        elif kind == "ChannelDelta":
+            mid, mix = m.project(x, step, v), m.scan
+        else:
+            return
+        sec = event_time(lambda: mix(mid, step, v), reps=5, warm=1)
+        key = f"{tag}_{kind}"
+        out[key + "_us"] = round(sec * 1e6, 1)
+        if nbytes is not None:
+            out[key + "_gbs"] = round(nbytes / sec / 1e9, 1)
+            out[key + "_frac"] = round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)
+        if flops is not None:
+            peak = MFMA_PEAK["bf16"] if kind in ("Attention", "LatentAttention") else MFMA_PEAK["fp32"]
+            out[key + "_tflops"] = round(flops / sec / 1e12, 2)
+            out[key + "_frac"] = round(flops / sec / peak, 4)
+
+    def state_bytes(view):
+        from burn_lm_amd.cache.cache import KVView
+        views = view if isinstance(view, tuple) else (view,)
+        kv = [v for v in views if isinstance(v, KVView)]
+        if kv:
+            n = kv[0].need
+            return batch * context * (n.n_kv_heads * n.head_dim + n.v_heads * n.v_dim) * kv[0].k.element_size()
+        return 2 * batch * max(v.tensor[0].numel() * v.tensor.element_size() for v in views)
+
+    slots = [engine.open() for _ in range(batch)]
+    for s in slots:
+        engine.cache.reserve([(s, context)])
+        engine.cache.advance(s, context - 1)
+    step = engine.build_step([(s, [1], [0]) for s in slots])
+    x = torch.randn(batch, width, device=rt.device).to(rt.dtype)
+    for kind, (block, view) in seen.items():
+        run(kind, block, view, step, x, "decode", nbytes=state_bytes(view))
+    for s in slots:
+        engine.close(s)
+    T = prefill_tokens
+    s = engine.open()
+    engine.cache.reserve([(s, T)])
+    step = engine.build_step([(s, [1] * T, [T - 1])])
+    x = torch.randn(T, width, device=rt.device).to(rt.dtype)
+    for kind, (block, view) in seen.items():
+        run(kind, block, view, step, x, "prefill", flops=block.mixer.mixing_flops(0, T))
+    engine.close(s)
+    return out
+
+
+def run_design(args):
+    """--design fuvirax: prompt and decode throughput of the design at sizes that resemble a real model's layers
+    (random weights), beside the Llama of equal size, and the mixing kernels of both alone against their limits."""
+    import torch
+    from burn_lm_amd.config.presets import preset
+    from burn_lm_amd.engine.loading import random_engine
+    from burn_lm_amd.sampling.sampler import Sampler
+    if args.design != "fuvirax":
+        print(f"bench.py: no design named {args.design!r}; known: fuvirax")
+        sys.exit(2)
+    layers = args.layers or 6
+    record = {"metric": "design_throughput", "design": args.design, "dtype": args.dtype, "data": "synthetic", "n_gpus": 1,
+              "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens, "layers": layers,
+              "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+    for name in (args.sizes.split(",") if args.sizes else DESIGN_SIZES):
+        size = DESIGN_SIZES[name]
+        base = preset(size["llama"])
+        base["num_hidden_layers"] = layers
+        configs = {"fuvirax": fuvirax_config(size["width"], size["ff"], size["heads"], layers, base["vocab_size"]),
+                   "llama": base}
+        entry = {}
+        for model, config in configs.items():
+            print(f"[bench] {name} {model}: building", file=sys.stderr, flush=True)
+            engine = random_engine(config, seed=0, dtype=args.dtype, max_tokens=args.batch * args.context,
+                                   max_seqs=args.batch, max_context=args.context, quick_weights=True)
+            pre = time_prefill(engine, args.prefill_tokens, reps=3)
+            c = engine.model.step_costs([0], [args.prefill_tokens], 1)
+            sec, med = time_decode(engine, Sampler(temperature=0.0), args.batch, args.context, args.steps, args.warmup)
+            roof = decode_roofline(engine, args.batch, args.context, args.steps, sec)
+            entry[model] = {"prefill_tokens_per_s": round(args.prefill_tokens / pre, 1), "prefill_ms": round(pre * 1e3, 3),
+                            "prefill_frac_of_bf16_peak": round(c["flops"] / pre / MFMA_PEAK["bf16"], 4),
+                            "decode_tokens_per_s": round(args.batch / sec, 1), "decode_ms_per_step": round(sec * 1e3, 4),
+                            "decode_step_ms_median": round(med * 1e3, 4), "decode_frac_of_hbm_peak": roof["frac"],
+                            "kernels": mixer_rates(engine, args.batch, args.context, args.prefill_tokens)}
+            del engine
+            torch.cuda.empty_cache()
+        record["sizes"][name] = entry
+    print(json.dumps(record))
+
+
 def run_unequal(args):
     """An unequal batch through the generation loop: --unequal N prompts of 64..2048 seeded random
     tokens in one prefill step, then --generate greedy tokens each.  One JSON line of its own."""
@@ -361,6 +490,11 @@ def main():
                          "step ten times, or (decode-loop, for counter runs, where every launch is slow) --steps decode steps "
                          "launched kernel by kernel on a cache that is filled without a prompt step; prints its time and "
                          "no JSON line, and says on stderr where it is")
+    ap.add_argument("--design", default=None, metavar="NAME",
+                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax) at model-like "
+                         "layer sizes beside the Llama of equal size, with the mixing kernels alone (--layers, default 6; "
+                         "--sizes 1b-like,3b-like)")
+    ap.add_argument("--sizes", default=None, help="with --design: which of its sizes, with commas between them")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this library has no multi-GPU path (run with --gpus 1)")
@@ -368,6 +502,8 @@ def main():
 
     if args.unequal:
         return run_unequal(args)
+    if args.design:
+        return run_design(args)
 
     from burn_lm_amd.config.presets import preset
     from burn_lm_amd.engine.loading import random_engine

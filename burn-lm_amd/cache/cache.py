@@ -252,6 +252,8 @@ class Cache:
             if isinstance(v, KVView):
                 keys = min(length, v.need.window) if v.need.window > 0 else length
                 total += (v.need.n_kv_heads * v.need.head_dim + v.need.v_heads * v.need.v_dim) * keys * v.k.element_size()
+            elif isinstance(v, StateView):      # fixed-size state is read and written once a step
+                total += 2 * v.tensor[0].numel() * v.tensor.element_size()
         return total
 
     def __del__(self):

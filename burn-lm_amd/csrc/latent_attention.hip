@@ -14,12 +14,13 @@
 // ---------------------------------------------------------------------------------------
 // down [T][ld_down]: R latent lanes then Dr key lanes.  q [T][ld_q], head h at h * (dn + Dr).  cos_sin [positions][half_t]
 // (cos, sin), of which the first rot/2 pairs turn lanes (i, i + rot/2) of the Dr part.
-// qabs [T][H][R + Dr] float gets the rotated query parts at lane R.
+// qabs [T][H][R + Dr] (float or the cache's type) gets the rotated query parts at lane R.  vcache (may be null):
+// pages [R][page] that receive the latent transposed, for the matrix-core attention.
 // ---------------------------------------------------------------------------------------
-template <typename TA>
+template <typename TA, typename TQ>
 __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, const TA* __restrict__ q, int ld_q, int H, int dn,
                                     const float* __restrict__ norm_w, float eps, const float2* __restrict__ cos_sin,
-                                    int half_t, int rot, float* __restrict__ qabs, TA* __restrict__ kcache,
+                                    int half_t, int rot, TQ* __restrict__ qabs, TA* __restrict__ kcache, TA* __restrict__ vcache,
                                     const int* __restrict__ positions, const int* __restrict__ token_seq,
                                     const int* __restrict__ block_table, int table_width, int page_size, int R, int Dr,
                                     int write_kv) {
@@ -41,7 +42,7 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
       const float other = to_float(src[d < half ? d + half : d - half]);
       v = d < half ? v * c.x - other * c.y : v * c.x + other * c.y;
     }
-    qabs[((size_t)t * H + h) * (R + Dr) + R + d] = v;
+    qabs[((size_t)t * H + h) * (R + Dr) + R + d] = from_float<TQ>(v);
   }
   const int page = block_table[(size_t)b * table_width + pos / page_size];
   if (!write_kv || page < 0) return;
@@ -53,7 +54,12 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
     ss += v * v;
   }
   const float inv = 1.0f / sqrtf(block_sum<true>(ss, red) / (float)R + eps);
-  for (int d = threadIdx.x; d < R; d += blockDim.x) dst[d] = from_float<TA>(to_float(row[d]) * inv * norm_w[d]);
+  TA* vdst = vcache ? vcache + (size_t)page * R * page_size + (pos % page_size) : nullptr;   // transposed page [R][page]
+  for (int d = threadIdx.x; d < R; d += blockDim.x) {
+    const TA c = from_float<TA>(to_float(row[d]) * inv * norm_w[d]);
+    dst[d] = c;
+    if (vdst) vdst[(size_t)d * page_size] = c;
+  }
   for (int d = threadIdx.x; d < Dr; d += blockDim.x) {
     float v = to_float(row[R + d]);
     if (d < rot) {
@@ -67,19 +73,20 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
 }
 
 extern "C" int blm_latent_write(const void* down, int ld_down, const void* q, int ld_q, int dtype, int T, int H, int dn,
-                                const float* norm_w, float eps, const void* cos_sin, int half_t, int rot, float* qabs,
-                                void* kcache, const int* positions, const int* token_seq, const int* block_table,
+                                const float* norm_w, float eps, const void* cos_sin, int half_t, int rot, void* qabs,
+                                int qabs_dtype, void* kcache, void* vcache, const int* positions, const int* token_seq, const int* block_table,
                                 int table_width, int page_size, int R, int Dr, int write_kv, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && H > 0 && dn >= 0 && R > 0 && Dr >= 0, "latent_write: bad sizes");
   BLM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= Dr && rot / 2 <= half_t, "latent_write: %d turning lanes do not fit %d", rot, Dr);
   BLM_REQUIRE(page_size > 0 && table_width > 0 && ld_down >= R + Dr && ld_q >= H * (dn + Dr), "latent_write: bad geometry");
-#define BLM_LW(TA)                                                                                                      \
-  hipLaunchKernelGGL(latent_write_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)down, ld_down, (const TA*)q, ld_q, H, \
-                     dn, norm_w, eps, (const float2*)cos_sin, half_t, rot, qabs, (TA*)kcache, positions, token_seq,     \
-                     block_table, table_width, page_size, R, Dr, write_kv)
-  if (dtype == BLM_F32) BLM_LW(float);
-  else if (dtype == BLM_BF16) BLM_LW(bf16);
-  else return blm_fail("latent_write: unsupported dtype %d", dtype);
+#define BLM_LW(TA, TQ)                                                                                                  \
+  hipLaunchKernelGGL((latent_write_kernel<TA, TQ>), dim3(T), dim3(256), 0, stream, (const TA*)down, ld_down, (const TA*)q, \
+                     ld_q, H, dn, norm_w, eps, (const float2*)cos_sin, half_t, rot, (TQ*)qabs, (TA*)kcache, (TA*)vcache,  \
+                     positions, token_seq, block_table, table_width, page_size, R, Dr, write_kv)
+  if (dtype == BLM_F32 && qabs_dtype == BLM_F32) BLM_LW(float, float);
+  else if (dtype == BLM_BF16 && qabs_dtype == BLM_F32) BLM_LW(bf16, float);
+  else if (dtype == BLM_BF16 && qabs_dtype == BLM_BF16) BLM_LW(bf16, bf16);
+  else return blm_fail("latent_write: unsupported dtypes %d / %d", dtype, qabs_dtype);
 #undef BLM_LW
   BLM_LAUNCH_CHECK("latent_write");
   return 0;
@@ -333,4 +340,254 @@ extern "C" int blm_latent_attn(const float* qabs, float* olat, int cache_dtype, 
     return blm_fail("latent_attn: unsupported dtype %d", cache_dtype);
   BLM_LAUNCH_CHECK("latent_attn");
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// The attention on the matrix cores (bfloat16 cache and queries, float softmax and accumulation).
+//
+// All heads share the cached rows, so the 16 "query columns" of a wavefront are 16 consecutive (token, head)
+// pairs of one sequence, each with its own position.  Per page of 64 rows:
+//   S^T = K Q^T      A = 16 cache rows x 32 lanes of [latent | key part] per instruction, B = Q^T; lane
+//                    (kg, c) gets the scores of column c for rows kg*4 .. kg*4+3 of each 16-row tile
+//   O^T += V^T P^T   A = 16 latent lanes x 32 rows from the transposed latent pages ([R][64] per page),
+//                    B = the probabilities the lane has just computed.  The rows of a page are dealt to the
+//                    four score tiles so that the eight rows a lane supplies are neighbours in the
+//                    transposed page (lat_key_of), as in this library's other matrix-core attention.
+// Fragments come straight from global memory (the pages of a sequence are shared by all its wavefronts and
+// stay in the caches); no shared memory, no barriers.  With n_splits > 1 the pages of a wavefront's columns
+// are cut into pieces whose partial results the last wavefront to arrive merges.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 lat_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float lat_f32x4;
+
+__device__ __forceinline__ constexpr int lat_key_of(int t, int i) { return (t >> 1) * 32 + (i >> 2) * 8 + (t & 1) * 4 + (i & 3); }
+
+// keep the first n (0..8) bf16 of a 16-byte group, zero the rest
+__device__ __forceinline__ uint4 lat_keep_first(uint4 v, int n) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int left = n - 2 * i;
+    w[i] = left >= 2 ? w[i] : (left == 1 ? (w[i] & 0xffffu) : 0u);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+#define LATM_WAVES 4
+template <int R, int DR>
+__global__ void __launch_bounds__(LATM_WAVES* BLM_WAVE)
+    latent_attn_mfma_kernel(const bf16* __restrict__ q, float* __restrict__ olat, const int* __restrict__ cu_seqlens,
+                            const int* __restrict__ lens_after, const int* __restrict__ block_table, int table_width,
+                            const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int B, int H,
+                            int tiles_per_seq, float scale2, int n_splits, float* part_o, float* part_ml, int* arrivals) {
+  constexpr int W = R + DR;
+  constexpr int KS = (W + 31) / 32;
+  constexpr int DT = R / 16;
+  static_assert(R % 16 == 0 && W % 8 == 0, "latent lanes in tiles of 16, rows in pieces of 16 bytes");
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const int tile_id = blockIdx.x * LATM_WAVES + wave;          // over sequences x tiles of 16 columns
+  const int b = tile_id / tiles_per_seq, tile = tile_id - b * tiles_per_seq;
+  if (b >= B) return;                                            // the last block's surplus wavefronts
+  const int split = blockIdx.y;
+  const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
+  const int n_cols = n_new * H;
+  if (tile * 16 >= n_cols) return;                               // also a padding sequence
+  const int after = lens_after[b];
+  const int past = after - n_new;
+  // this lane's column
+  const int idx = tile * 16 + c;
+  const bool valid = idx < n_cols;
+  const int tok = valid ? idx / H : 0, head = valid ? idx - tok * H : 0;
+  const int qpos = valid ? past + tok : -1;
+  const size_t item = (size_t)(t_first + tok) * H + head;
+  // the last column of the tile sees the most
+  const int last_idx = min(tile * 16 + 15, n_cols - 1);
+  const int max_qpos = past + last_idx / H;
+  const int max_key = after - 1;
+  const int n_pages = max_qpos / 64 + 1;
+  const int per = (n_pages + n_splits - 1) / n_splits;
+  const int p_begin = split * per, p_end = min(n_pages, p_begin + per);
+  const int* bt = block_table + (size_t)b * table_width;
+
+  uint4 qf[KS];
+  {
+    const bf16* qrow = q + item * W;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + kg * 8;
+      qf[ks] = (valid && (W % 32 == 0 || d < W)) ? *reinterpret_cast<const uint4*>(qrow + d) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  float m = -INFINITY;
+  lat_f32x4 l = {0.f, 0.f, 0.f, 0.f};
+  lat_f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int pi = p_begin; pi < p_end; ++pi) {
+    const int page = bt[pi];
+    const int key0 = pi * 64;
+    const bf16* kp = kcache + (size_t)page * 64 * W;
+    const bf16* vp = vcache + (size_t)page * R * 64;
+    float s[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bf16* krow = kp + (size_t)lat_key_of(t, c) * W;
+      uint4 kf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + kg * 8;
+        kf[ks] = (W % 32 == 0 || d < W) ? *reinterpret_cast<const uint4*>(krow + d) : make_uint4(0u, 0u, 0u, 0u);
+      }
+      lat_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, kf[ks]),
+                                                      __builtin_bit_cast(lat_bf16x8, qf[ks]), acc, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kj = key0 + lat_key_of(t, kg * 4 + r);
+        s[t][r] = kj <= qpos ? acc[r] : -INFINITY;      // whatever the rows past the data hold, it is replaced here
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = blm_max(mx, s[t][r]);
+    mx = rows_max(mx);
+    const float m_new = blm_max(m, mx * scale2);
+    const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        s[t][r] = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
+    if (__any(m != m_new)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[dt][r] *= corr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) l[r] *= corr;
+    }
+    m = m_new;
+    const bool tail = key0 + 63 > max_key;       // the page holds places past the data: 0 * garbage must stay 0
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 pf;
+      pf.x = f32x2_to_bf16x2_bits(s[2 * h][0], s[2 * h][1]);
+      pf.y = f32x2_to_bf16x2_bits(s[2 * h][2], s[2 * h][3]);
+      pf.z = f32x2_to_bf16x2_bits(s[2 * h + 1][0], s[2 * h + 1][1]);
+      pf.w = f32x2_to_bf16x2_bits(s[2 * h + 1][2], s[2 * h + 1][3]);
+      // the softmax's denominator: a row of ones in place of V^T sums the rounded probabilities of every column
+      l = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          __builtin_bit_cast(lat_bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u)),
+          __builtin_bit_cast(lat_bf16x8, pf), l, 0, 0, 0);
+      const int keep = max_key - (key0 + h * 32 + kg * 8) + 1;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        uint4 va = *reinterpret_cast<const uint4*>(vp + (size_t)(dt * 16 + c) * 64 + h * 32 + kg * 8);
+        if (tail) va = lat_keep_first(va, keep);
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, va),
+                                                        __builtin_bit_cast(lat_bf16x8, pf), o[dt], 0, 0, 0);
+      }
+    }
+  }
+  float* orow = olat + item * R;
+  if (n_splits == 1) {
+    if (valid) {
+      const float inv = 1.0f / l[0];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<float4*>(orow + dt * 16 + kg * 4) = make_float4(o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv);
+    }
+    return;
+  }
+  // publish this piece: per column its maximum, sum and unnormalised result
+  const size_t gcol = (size_t)tile_id * 16 + c;
+  float* po = part_o + (gcol * n_splits + split) * R;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      __hip_atomic_store(po + dt * 16 + kg * 4 + r, o[dt][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (kg == 0) {
+    __hip_atomic_store(part_ml + (gcol * n_splits + split) * 2, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part_ml + (gcol * n_splits + split) * 2 + 1, l[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the wavefront's stores have been acknowledged
+  int last = 0;
+  if (lane == 0) {
+    const int before = __hip_atomic_fetch_add(arrivals + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = before == n_splits - 1;
+    if (last) __hip_atomic_store(arrivals + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  last = __shfl(last, 0, BLM_WAVE);
+  if (!last || !valid) return;
+  float M = -INFINITY, L = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < n_splits; ++sp) {
+    const float* ml = part_ml + (gcol * n_splits + sp) * 2;
+    const float ms = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float ls = __hip_atomic_load(ml + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ls == 0.f) continue;
+    const float Mn = fmaxf(M, ms);
+    const float keep = __builtin_amdgcn_exp2f(M - Mn), take = __builtin_amdgcn_exp2f(ms - Mn);
+    L = L * keep + ls * take;
+    const float* ps = part_o + (gcol * n_splits + sp) * R;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        o[dt][r] = o[dt][r] * keep + __hip_atomic_load(ps + dt * 16 + kg * 4 + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * take;
+    M = Mn;
+  }
+  const float inv = 1.0f / L;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    *reinterpret_cast<float4*>(orow + dt * 16 + kg * 4) = make_float4(o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv);
+}
+
+// the sizes the matrix-core form is built for (latent lanes, turned key lanes)
+#define BLM_LATM_SIZES(X) X(512, 64) X(256, 64) X(256, 32) X(128, 64) X(128, 32) X(64, 32) X(64, 16) X(32, 16)
+
+extern "C" int blm_latent_attn_mfma_supported(int R, int Dr) {
+#define BLM_LATM_HAS(r, d) if (R == r && Dr == d) return 1;
+  BLM_LATM_SIZES(BLM_LATM_HAS)
+#undef BLM_LATM_HAS
+  return 0;
+}
+
+// q: bfloat16 [T][H][R + Dr]; olat float [T][H][R]; key pages [pages][1][64][R + Dr], transposed latent pages
+// [pages][1][R][64], both bfloat16.  B sequences of at most max_new tokens.  Workspace for n_splits > 1:
+// part_o (B * tiles * 16 * n_splits * R floats), part_ml (... * 2), arrivals (B * tiles ints, zero and left zero),
+// with tiles = ceil(max_new * H / 16).
+extern "C" int blm_latent_attn_mfma(const void* q, float* olat, const int* cu_seqlens, const int* lens_after,
+                                    const int* block_table, int table_width, const void* kcache, const void* vcache,
+                                    int page_size, int B, int max_new, int H, int R, int Dr, float scale, int n_splits,
+                                    float* part_o, float* part_ml, int* arrivals, hipStream_t stream) {
+  BLM_REQUIRE(B > 0 && max_new > 0 && H > 0, "latent_attn_mfma: bad sizes B=%d max_new=%d H=%d", B, max_new, H);
+  BLM_REQUIRE(page_size == 64 && table_width > 0, "latent_attn_mfma: pages of 64 rows");
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml && arrivals)),
+              "latent_attn_mfma: %d splits need their workspace", n_splits);
+  const long long tiles = ((long long)max_new * H + 15) / 16;
+  const long long waves = (long long)B * tiles;
+  BLM_REQUIRE(waves < 2147483647LL, "latent_attn_mfma: too many tiles");
+  const unsigned blocks = (unsigned)((waves + LATM_WAVES - 1) / LATM_WAVES);
+  const float scale2 = scale * 1.4426950408889634f;
+  dim3 grid(blocks, (unsigned)n_splits);
+#define BLM_LATM_CASE(r, d)                                                                                            \
+  if (R == r && Dr == d) {                                                                                             \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<r, d>), grid, dim3(LATM_WAVES * BLM_WAVE), 0, stream, (const bf16*)q,  \
+                       olat, cu_seqlens, lens_after, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache, \
+                       B, H, (int)tiles, scale2, n_splits, part_o, part_ml, arrivals);                                 \
+    BLM_LAUNCH_CHECK("latent_attn_mfma");                                                                              \
+    return 0;                                                                                                          \
+  }
+  BLM_LATM_SIZES(BLM_LATM_CASE)
+#undef BLM_LATM_CASE
+  return blm_fail("latent_attn_mfma: a latent of %d + %d lanes is not among the sizes it is built for", R, Dr);
 }

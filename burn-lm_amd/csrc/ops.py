@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 _lib = None
 _lock = threading.Lock()
 
@@ -32,8 +32,12 @@ _SIGNATURES = {
                         _c_int, _c_int, _c_void_p],
     "blm_xielu": [_c_void_p, _c_void_p, _c_int, ctypes.c_longlong, _c_float, _c_float, _c_void_p],
     "blm_latent_write": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_void_p,
-                         _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                         _c_int, _c_int, _c_void_p],
+                         _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                         _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_latent_attn_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p],
+    "blm_latent_attn_mfma_supported": [_c_int, _c_int],
     "blm_head_project": [_c_void_p, _c_int, ctypes.c_longlong, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
                          ctypes.c_longlong, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_latent_attn": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int,
@@ -841,16 +845,22 @@ def xielu(z, out, a_pos, a_neg):
 # ------------------------------------------------------------------------------------------
 # attention over a shared latent
 def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_table, page_size, H, dn, R, Dr,
-                 write_kv=True):
+                 write_kv=True, vcache=None):
     """down [T, >= R + Dr]: latent lanes then the shared key lanes; q [T, H * (dn + Dr)].  The latent is RMS-normed
     (norm_w, eps), the first `rot` of the Dr key lanes are turned by the token's position (pairs half of rot
     apart; cos_sin float32 [positions, n, 2]), and the row [latent | key lanes] goes into the token's place of the
     key pages [pages, 1, page, R + Dr].  The queries' Dr lanes are turned alike into qabs[:, :, R:] (float32
-    [T, H, R + Dr])."""
-    _gpu(down, q, norm_w, cos_sin, qabs, kcache, block_table)
+    [T, H, R + Dr], or the cache's dtype).  vcache: pages [pages, 1, R, page] that get the latent transposed."""
+    _gpu(down, q, norm_w, cos_sin, qabs, kcache, block_table, vcache)
     T = down.shape[0]
     _contig("cos_sin", cos_sin); _contig("kcache", kcache); _contig("qabs", qabs)
-    _f32("norm_w", norm_w, R); _f32("qabs", qabs, T * H * (R + Dr))
+    _f32("norm_w", norm_w, R)
+    if qabs.numel() != T * H * (R + Dr) or qabs.dtype not in (torch.float32, kcache.dtype):
+        raise KernelError("latent_write: qabs is [T, H, R + Dr] in float32 or the cache's dtype")
+    if vcache is not None:
+        _contig("vcache", vcache)
+        if tuple(vcache.shape) != (kcache.shape[0], 1, R, page_size) or vcache.dtype != kcache.dtype:
+            raise KernelError(f"latent_write: transposed latent pages {tuple(vcache.shape)} do not fit")
     if down.stride(1) != 1 or q.stride(1) != 1 or down.dtype != q.dtype or kcache.dtype != q.dtype:
         raise KernelError("latent_write: down, q and the cache must share a dtype, rows contiguous")
     if tuple(q.shape) != (T, H * (dn + Dr)) or tuple(kcache.shape[1:]) != (1, page_size, R + Dr):
@@ -859,8 +869,8 @@ def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_t
         raise KernelError("latent_write: cos_sin must be float32 [positions, pairs, 2] and cover the step's positions")
     _i32("block_table", block_table)
     _call("blm_latent_write", down.data_ptr(), down.stride(0), q.data_ptr(), q.stride(0), _code(q), T, H, dn, norm_w.data_ptr(),
-          float(eps), cos_sin.data_ptr(), cos_sin.shape[1], rot, qabs.data_ptr(), kcache.data_ptr(),
-          step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+          float(eps), cos_sin.data_ptr(), cos_sin.shape[1], rot, qabs.data_ptr(), _code(qabs), kcache.data_ptr(),
+          _ptr(vcache), step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
           R, Dr, 1 if write_kv else 0, _stream())
 
 
@@ -925,6 +935,45 @@ def latent_attn(qabs, olat, kcache, step, block_table, page_size, H, R, Dr, scal
     _call("blm_latent_attn", qabs.data_ptr(), olat.data_ptr(), _code(kcache), step.positions.data_ptr(),
           step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), page_size, T, H, R,
           Dr, float(scale), n_splits, _ptr(part_o), _ptr(part_ml), _ptr(arrivals), _stream())
+    return olat
+
+
+def latent_attn_mfma_supported(dtype, R, Dr, page_size=64):
+    return dtype == torch.bfloat16 and page_size == 64 and bool(library().blm_latent_attn_mfma_supported(R, Dr))
+
+
+def latent_attn_mfma_max_splits(n_seqs, max_new, H, R):
+    """Most pieces the matrix-core form can cut the pages into for a step of this shape."""
+    waves = n_seqs * ((max_new * H + 15) // 16)
+    if waves > ARRIVAL_COUNTERS:
+        return 1
+    return max(1, LATENT_SCRATCH_FLOATS // (waves * 16 * (R + 2)))
+
+
+def latent_attn_mfma(q, olat, kcache, vcache, step, block_table, page_size, H, R, Dr, scale, n_splits=1):
+    """The same function as latent_attn on the matrix cores: q bfloat16 [T, H, R + Dr], key pages and transposed
+    latent pages ([pages, 1, R, 64]) in bfloat16; olat float32 [T, H, R]."""
+    _gpu(q, olat, kcache, vcache, block_table)
+    T = q.shape[0]
+    _contig("q", q); _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
+    _f32("olat", olat, T * H * R)
+    if q.dtype != torch.bfloat16 or kcache.dtype != torch.bfloat16 or vcache.dtype != torch.bfloat16 or q.numel() != T * H * (R + Dr):
+        raise KernelError("latent_attn_mfma: queries [T, H, R + Dr] and both kinds of pages in bfloat16")
+    if tuple(kcache.shape[1:]) != (1, page_size, R + Dr) or tuple(vcache.shape) != (kcache.shape[0], 1, R, page_size):
+        raise KernelError(f"latent_attn_mfma: pages {tuple(kcache.shape)} / {tuple(vcache.shape)} do not fit")
+    if T != step.n_tokens or step.cu_seqlens.numel() < step.n_seqs + 1 or block_table.shape[0] < step.n_seqs:
+        raise KernelError("latent_attn_mfma: the step's index arrays do not fit the queries")
+    part_o = part_ml = arrivals = None
+    if n_splits > 1:
+        if n_splits > latent_attn_mfma_max_splits(step.n_seqs, step.max_new, H, R):
+            raise KernelError("latent_attn_mfma: more pieces than the workspace holds (see latent_attn_mfma_max_splits)")
+        cols = step.n_seqs * ((step.max_new * H + 15) // 16) * 16
+        buf = latent_attn_init(q.device)
+        part_o, part_ml = buf[: cols * n_splits * R], buf[cols * n_splits * R: cols * n_splits * (R + 2)]
+        arrivals = arrival_counters(q.device)
+    _call("blm_latent_attn_mfma", q.data_ptr(), olat.data_ptr(), step.cu_seqlens.data_ptr(), step.lens_after.data_ptr(),
+          block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(), page_size, step.n_seqs,
+          step.max_new, H, R, Dr, float(scale), n_splits, _ptr(part_o), _ptr(part_ml), _ptr(arrivals), _stream())
     return olat
 
 

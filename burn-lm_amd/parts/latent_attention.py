@@ -9,11 +9,14 @@ function, so the cache holds one row of kv_rank + rot_dim lanes per token for al
 Rotation: lane i of the first ``rot_dims`` turned lanes pairs with lane i + rot_dims/2."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .base import KVNeed, Mixer, TensorSpec
 
 DECODE_BLOCKS_PER_UNIT = 2     # blocks of four (token, head) wavefronts the split decode aims for per compute unit
+MFMA_MAX_PIECES = 64           # most pieces the matrix-core decode cuts a sequence's pages into
 
 
 class LatentAttention(Mixer):
@@ -29,7 +32,11 @@ class LatentAttention(Mixer):
                 n["o"]: TensorSpec((d, H * dv))}
 
     def cache_need(self):
+        """One row [latent | turned key part] per token for all heads.  Where the matrix-core attention runs
+        (bfloat16, sizes it is built for) the latent is kept a second time, transposed, as the value pages."""
         p = self.params
+        if getattr(self, "use_mfma", False):
+            return KVNeed(1, p["kv_rank"] + p["rot_dim"], 0, value_dim=p["kv_rank"])
         return KVNeed(1, p["kv_rank"] + p["rot_dim"], 0, no_values=True)
 
     def bind(self, tensors, rt):
@@ -51,6 +58,8 @@ class LatentAttention(Mixer):
         self.w_uv = tensors[n["uv"]].view(H, dv, R).contiguous()
         self.w_o = rt.weight(tensors[n["o"]])
         rt.ops.latent_attn_init(rt.device)
+        self.use_mfma = (os.environ.get("BURN_LM_AMD_LATENT_MFMA") != "0" and self.w_uk_t.dtype == torch.bfloat16
+                         and rt.ops.latent_attn_mfma_supported(rt.dtype, R, self.dr))
 
     def step_bytes(self, rows):
         return sum(w.numel() * w.element_size() for w in (self.w_in.w, self.w_o.w, self.w_uk_t, self.w_uv))
@@ -74,9 +83,11 @@ class LatentAttention(Mixer):
         T = x.shape[0]
         qd = rt.linear(x, self.w_in)                         # [T, H (dn + dr) | R + dr]
         q, down = qd[:, :self.n_q], qd[:, self.n_q:]
-        qabs = torch.empty(T, H, R + dr, dtype=torch.float32, device=x.device)
+        mfma = self.use_mfma and view.v.numel() > 0 and view.page_size == 64
+        qabs = torch.empty(T, H, R + dr, dtype=rt.dtype if mfma else torch.float32, device=x.device)
         ops.latent_write(down, q, self.norm_w, self.eps, self.position.table, self.rot, qabs, view.k, step,
-                         view.block_table(step), view.page_size, H, dn, R, dr, write_kv=view.store)
+                         view.block_table(step), view.page_size, H, dn, R, dr, write_kv=view.store,
+                         vcache=view.v if mfma else None)
         ops.head_project(q, dn + dr, self.w_uk_t, qabs.view(T, H * (R + dr)), R + dr)
         return qabs
 
@@ -87,6 +98,14 @@ class LatentAttention(Mixer):
         T = qabs.shape[0]
         olat = torch.empty(T, H, R, dtype=torch.float32, device=qabs.device)
         n_splits = 1
+        if qabs.dtype == torch.bfloat16:        # the matrix-core form: one wavefront per 16 (token, head) pairs
+            if step.max_new == 1:
+                waves = step.n_seqs * ((H + 15) // 16)
+                pages = (step.max_len_after + 63) // 64
+                n_splits = max(1, min(pages, (4 * rt.compute_units) // waves, MFMA_MAX_PIECES,
+                                      ops.latent_attn_mfma_max_splits(step.n_seqs, 1, H, R)))
+            return ops.latent_attn_mfma(qabs, olat, view.k, view.v, step, view.block_table(step), view.page_size, H, R,
+                                        dr, self.scale, n_splits)
         if step.max_new == 1:
             chunks = (step.max_len_after + 63) // 64
             blocks = (T * H + 3) // 4

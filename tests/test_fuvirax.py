@@ -46,7 +46,9 @@ def config(layers, width=48, vocab=101, streams=3, loop=None, logit_scale=0.7, e
     return c
 
 
-MIXED = config([latent(), hgrn(), delta(), latent(heads=2, dim=16, rot_dim=4, vdim=8, kv_rank=16, ff=None), hgrn(ff=None)],
+# the first attention layer has a latent of a size only the generic kernel takes, the second one of a size the
+# matrix-core kernel is built for (in bfloat16 runs)
+MIXED = config([latent(), hgrn(), delta(), latent(heads=2, dim=16, rot_dim=16, vdim=8, kv_rank=32, ff=None), hgrn(ff=None)],
                loop=(1, 3, 2))
 # sizes that are no multiples of eight, one stream, one query/key head, two taps, no loop
 ODD = config([latent(heads=3, dim=12, rot_dim=6, vdim=10, kv_rank=20, ff=50), hgrn(heads=3, dim=10, vdim=12, ff=50),
@@ -233,8 +235,11 @@ def whole(eng, toks):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("layer", [latent(ff=None), hgrn(ff=None), delta(ff=None), delta(heads=2, kv_heads=2, conv=1, ff=None),
-                                   latent(heads=5, dim=4, rot_dim=12, vdim=4, kv_rank=12, ff=40)],
-                         ids=["latent", "hgrn2", "delta", "delta_one_tap", "latent_with_ff"])
+                                   latent(heads=5, dim=4, rot_dim=12, vdim=4, kv_rank=12, ff=40),
+                                   latent(heads=5, dim=8, rot_dim=16, vdim=8, kv_rank=64, ff=None),
+                                   latent(heads=20, dim=8, rot_dim=32, vdim=4, kv_rank=64, ff=None)],
+                         ids=["latent", "hgrn2", "delta", "delta_one_tap", "latent_with_ff", "latent_matrix_core_sizes",
+                              "latent_more_heads_than_a_tile"])
 def test_every_mixer_alone(tmp_path, layer, dtype):
     cfg = config([layer], streams=2)
     w = make_weights(cfg, 3)
@@ -363,6 +368,50 @@ def test_one_row_far_back_stands_out(dtype, n_splits):
         assert p[target, 1] > 0.99
         assert (olat[0].double().cpu() - want).abs().max() <= 1e-5, target
         assert (olat[0, 1].double().cpu() - row[:R].double()).abs().max() < 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_splits", [1, 3, 11])
+def test_one_row_far_back_stands_out_on_the_matrix_cores(n_splits):
+    """The same for the matrix-core kernel: two sequences of one token each (decoding), 20 heads (two tiles of
+    columns, the second partly empty), the latent also in its transposed pages; rows past the data hold NaN."""
+    from burn_lm_amd.csrc import ops
+    from burn_lm_amd.engine.batch import Step
+    dev, R, Dr, H, page = torch.device("cuda:0"), 64, 16, 20, 64
+    ops.latent_attn_init(dev)
+    g = torch.Generator().manual_seed(1)
+    lens = [701, 130]
+    pools = torch.randperm(24, generator=g).int()
+    tables = torch.full((2, 11), -1, dtype=torch.int32)
+    tables[0, :11], tables[1, :3] = pools[:11], pools[11:14]
+    q = torch.randn(2, H, R + Dr, generator=g)
+    q = (q / q.norm(dim=-1, keepdim=True)).bfloat16()
+    i32 = lambda a: torch.tensor(a, dtype=torch.int32, device=dev)
+    step = Step(n_tokens=2, n_seqs=2, n_wanted=0, token_ids=None, positions=i32([700, 129]), token_seq=i32([0, 1]),
+                seq_slots=i32([0, 1]), cu_seqlens=i32([0, 1, 2]), lens_after=i32(lens), want_rows=None, max_new=1,
+                max_len_after=701, max_position=700)
+    for target in (0, 63, 64, 127, 128, 129):
+        k = (torch.randn(24, 1, page, R + Dr, generator=g) * 0.05).bfloat16()
+        for b in range(2):       # places past each sequence's data: NaN
+            last_page, used = tables[b][(lens[b] - 1) // page], (lens[b] - 1) % page + 1
+            k[last_page, 0, used:] = float("nan")
+        rows = []
+        for b in range(2):
+            row = (q[b, 7].float() * 6.0).bfloat16()
+            k[tables[b][target // page], 0, target % page] = row
+            rows.append(row)
+        v = k[:, :, :, :R].transpose(2, 3).contiguous()
+        olat = torch.empty(2, H, R, dtype=torch.float32, device=dev)
+        ops.latent_attn_mfma(q.to(dev), olat, k.to(dev), v.to(dev), step, tables.to(dev), page, H, R, Dr, 8.0, n_splits)
+        torch.cuda.synchronize()
+        for b in range(2):
+            ctx = torch.cat([k[p, 0] for p in tables[b][: (lens[b] + page - 1) // page]]).double()[:lens[b]]
+            p = torch.softmax((ctx @ q[b].double().T) * 8.0, dim=0)
+            want = p.T @ ctx[:, :R]
+            assert p[target, 7] > 0.99
+            # probabilities go through bfloat16 on their way into the second product
+            assert (olat[b].double().cpu() - want).abs().max() <= 4e-3, (target, b)
+            assert (olat[b, 7].double().cpu() - rows[b][:R].double()).abs().max() < 0.05
 
 
 @pytest.mark.gpu
