@@ -348,7 +348,13 @@ def mixer_rates(engine, batch, context, prefill_tokens):
             mid, mix = m.project(x, step, v), m.scan
         else:
             return
-        sec = event_time(lambda: mix(mid, step, v), reps=5, warm=1)
+        mix(mid, step, v)          # once outside the recording
+        torch.cuda.synchronize()
+        g, n_rec = torch.cuda.CUDAGraph(), 4
+        with torch.cuda.graph(g):
+            for _ in range(n_rec):
+                mix(mid, step, v)
+        sec = event_time(g.replay, reps=5, warm=1) / n_rec
         key = f"{tag}_{kind}"
         out[key + "_us"] = round(sec * 1e6, 1)
         if nbytes is not None:

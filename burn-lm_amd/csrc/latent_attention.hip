@@ -355,7 +355,7 @@ extern "C" int blm_latent_attn(const float* qabs, float* olat, int cache_dtype, 
 //                    transposed page (lat_key_of), as in this library's other matrix-core attention.
 // Fragments come straight from global memory (the pages of a sequence are shared by all its wavefronts and
 // stay in the caches); no shared memory, no barriers.  With n_splits > 1 the pages of a wavefront's columns
-// are cut into pieces whose partial results the last wavefront to arrive merges.
+// are cut into pieces whose partial results a second kernel adds up.
 // ---------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 lat_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float lat_f32x4;
@@ -379,7 +379,7 @@ __global__ void __launch_bounds__(LATM_WAVES* BLM_WAVE)
     latent_attn_mfma_kernel(const bf16* __restrict__ q, float* __restrict__ olat, const int* __restrict__ cu_seqlens,
                             const int* __restrict__ lens_after, const int* __restrict__ block_table, int table_width,
                             const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int B, int H,
-                            int tiles_per_seq, float scale2, int n_splits, float* part_o, float* part_ml, int* arrivals) {
+                            int tiles_per_seq, float scale2, int n_splits, float* part_o, float* part_ml) {
   constexpr int W = R + DR;
   constexpr int KS = (W + 31) / 32;
   constexpr int DT = R / 16;
@@ -505,50 +505,45 @@ __global__ void __launch_bounds__(LATM_WAVES* BLM_WAVE)
     }
     return;
   }
-  // publish this piece: per column its maximum, sum and unnormalised result
+  // leave this piece: per column its maximum, sum and unnormalised result; latent_merge_kernel adds the pieces up
   const size_t gcol = (size_t)tile_id * 16 + c;
   float* po = part_o + (gcol * n_splits + split) * R;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      __hip_atomic_store(po + dt * 16 + kg * 4 + r, o[dt][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *reinterpret_cast<float4*>(po + dt * 16 + kg * 4) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
   if (kg == 0) {
-    __hip_atomic_store(part_ml + (gcol * n_splits + split) * 2, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(part_ml + (gcol * n_splits + split) * 2 + 1, l[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    part_ml[(gcol * n_splits + split) * 2] = m;
+    part_ml[(gcol * n_splits + split) * 2 + 1] = l[0];
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the wavefront's stores have been acknowledged
-  int last = 0;
-  if (lane == 0) {
-    const int before = __hip_atomic_fetch_add(arrivals + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    last = before == n_splits - 1;
-    if (last) __hip_atomic_store(arrivals + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  last = __shfl(last, 0, BLM_WAVE);
-  if (!last || !valid) return;
-  float M = -INFINITY, L = 0.f;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int sp = 0; sp < n_splits; ++sp) {
-    const float* ml = part_ml + (gcol * n_splits + sp) * 2;
-    const float ms = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const float ls = __hip_atomic_load(ml + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (ls == 0.f) continue;
-    const float Mn = fmaxf(M, ms);
-    const float keep = __builtin_amdgcn_exp2f(M - Mn), take = __builtin_amdgcn_exp2f(ms - Mn);
-    L = L * keep + ls * take;
-    const float* ps = part_o + (gcol * n_splits + sp) * R;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        o[dt][r] = o[dt][r] * keep + __hip_atomic_load(ps + dt * 16 + kg * 4 + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * take;
-    M = Mn;
-  }
+}
+
+// The pieces of a split run added up, one wavefront per column (a (token, head) pair): maxima in base 2.
+__global__ void __launch_bounds__(BLM_WAVE)
+    latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, float* __restrict__ olat,
+                        const int* __restrict__ cu_seqlens, int H, int R, int tiles_per_seq, int n_splits) {
+  const int gcol = blockIdx.x, lane = threadIdx.x;
+  const int per_seq = tiles_per_seq * 16;
+  const int b = gcol / per_seq, idx = gcol - b * per_seq;
+  const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
+  if (idx >= n_new * H) return;
+  const int tok = idx / H, head = idx - tok * H;
+  float* orow = olat + ((size_t)(t_first + tok) * H + head) * R;
+  const float* ml = part_ml + (size_t)gcol * n_splits * 2;
+  float M = -INFINITY;
+  for (int sp = 0; sp < n_splits; ++sp)
+    if (ml[sp * 2 + 1] != 0.f) M = fmaxf(M, ml[sp * 2]);
+  float L = 0.f;
+  for (int sp = 0; sp < n_splits; ++sp)
+    if (ml[sp * 2 + 1] != 0.f) L += ml[sp * 2 + 1] * __builtin_amdgcn_exp2f(ml[sp * 2] - M);
   const float inv = 1.0f / L;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-    *reinterpret_cast<float4*>(orow + dt * 16 + kg * 4) = make_float4(o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv);
+  for (int d = lane; d < R; d += BLM_WAVE) {
+    float acc = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+      const float ls = ml[sp * 2 + 1];
+      if (ls != 0.f) acc = fmaf(part_o[((size_t)gcol * n_splits + sp) * R + d], __builtin_amdgcn_exp2f(ml[sp * 2] - M), acc);
+    }
+    orow[d] = acc * inv;
+  }
 }
 
 // the sizes the matrix-core form is built for (latent lanes, turned key lanes)
@@ -563,15 +558,14 @@ extern "C" int blm_latent_attn_mfma_supported(int R, int Dr) {
 
 // q: bfloat16 [T][H][R + Dr]; olat float [T][H][R]; key pages [pages][1][64][R + Dr], transposed latent pages
 // [pages][1][R][64], both bfloat16.  B sequences of at most max_new tokens.  Workspace for n_splits > 1:
-// part_o (B * tiles * 16 * n_splits * R floats), part_ml (... * 2), arrivals (B * tiles ints, zero and left zero),
-// with tiles = ceil(max_new * H / 16).
+// part_o (B * tiles * 16 * n_splits * R floats), part_ml (... * 2), with tiles = ceil(max_new * H / 16).
 extern "C" int blm_latent_attn_mfma(const void* q, float* olat, const int* cu_seqlens, const int* lens_after,
                                     const int* block_table, int table_width, const void* kcache, const void* vcache,
                                     int page_size, int B, int max_new, int H, int R, int Dr, float scale, int n_splits,
-                                    float* part_o, float* part_ml, int* arrivals, hipStream_t stream) {
+                                    float* part_o, float* part_ml, hipStream_t stream) {
   BLM_REQUIRE(B > 0 && max_new > 0 && H > 0, "latent_attn_mfma: bad sizes B=%d max_new=%d H=%d", B, max_new, H);
   BLM_REQUIRE(page_size == 64 && table_width > 0, "latent_attn_mfma: pages of 64 rows");
-  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml && arrivals)),
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml)),
               "latent_attn_mfma: %d splits need their workspace", n_splits);
   const long long tiles = ((long long)max_new * H + 15) / 16;
   const long long waves = (long long)B * tiles;
@@ -583,8 +577,13 @@ extern "C" int blm_latent_attn_mfma(const void* q, float* olat, const int* cu_se
   if (R == r && Dr == d) {                                                                                             \
     hipLaunchKernelGGL((latent_attn_mfma_kernel<r, d>), grid, dim3(LATM_WAVES * BLM_WAVE), 0, stream, (const bf16*)q,  \
                        olat, cu_seqlens, lens_after, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache, \
-                       B, H, (int)tiles, scale2, n_splits, part_o, part_ml, arrivals);                                 \
+                       B, H, (int)tiles, scale2, n_splits, part_o, part_ml);                                           \
     BLM_LAUNCH_CHECK("latent_attn_mfma");                                                                              \
+    if (n_splits > 1) {                                                                                                \
+      hipLaunchKernelGGL(latent_merge_kernel, dim3((unsigned)(waves * 16)), dim3(BLM_WAVE), 0, stream, part_o, part_ml, \
+                         olat, cu_seqlens, H, R, (int)tiles, n_splits);                                                \
+      BLM_LAUNCH_CHECK("latent_merge");                                                                                \
+    }                                                                                                                  \
     return 0;                                                                                                          \
   }
   BLM_LATM_SIZES(BLM_LATM_CASE)

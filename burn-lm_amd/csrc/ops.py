@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 _lib = None
 _lock = threading.Lock()
 
@@ -35,8 +35,7 @@ _SIGNATURES = {
                          _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                          _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_latent_attn_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
-                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p,
-                             _c_void_p],
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_latent_attn_mfma_supported": [_c_int, _c_int],
     "blm_head_project": [_c_void_p, _c_int, ctypes.c_longlong, _c_int, _c_void_p, _c_int, _c_void_p, _c_int,
                          ctypes.c_longlong, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -945,8 +944,6 @@ def latent_attn_mfma_supported(dtype, R, Dr, page_size=64):
 def latent_attn_mfma_max_splits(n_seqs, max_new, H, R):
     """Most pieces the matrix-core form can cut the pages into for a step of this shape."""
     waves = n_seqs * ((max_new * H + 15) // 16)
-    if waves > ARRIVAL_COUNTERS:
-        return 1
     return max(1, LATENT_SCRATCH_FLOATS // (waves * 16 * (R + 2)))
 
 
@@ -963,17 +960,16 @@ def latent_attn_mfma(q, olat, kcache, vcache, step, block_table, page_size, H, R
         raise KernelError(f"latent_attn_mfma: pages {tuple(kcache.shape)} / {tuple(vcache.shape)} do not fit")
     if T != step.n_tokens or step.cu_seqlens.numel() < step.n_seqs + 1 or block_table.shape[0] < step.n_seqs:
         raise KernelError("latent_attn_mfma: the step's index arrays do not fit the queries")
-    part_o = part_ml = arrivals = None
+    part_o = part_ml = None
     if n_splits > 1:
         if n_splits > latent_attn_mfma_max_splits(step.n_seqs, step.max_new, H, R):
             raise KernelError("latent_attn_mfma: more pieces than the workspace holds (see latent_attn_mfma_max_splits)")
         cols = step.n_seqs * ((step.max_new * H + 15) // 16) * 16
         buf = latent_attn_init(q.device)
         part_o, part_ml = buf[: cols * n_splits * R], buf[cols * n_splits * R: cols * n_splits * (R + 2)]
-        arrivals = arrival_counters(q.device)
     _call("blm_latent_attn_mfma", q.data_ptr(), olat.data_ptr(), step.cu_seqlens.data_ptr(), step.lens_after.data_ptr(),
           block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(), page_size, step.n_seqs,
-          step.max_new, H, R, Dr, float(scale), n_splits, _ptr(part_o), _ptr(part_ml), _ptr(arrivals), _stream())
+          step.max_new, H, R, Dr, float(scale), n_splits, _ptr(part_o), _ptr(part_ml), _stream())
     return olat
 
 

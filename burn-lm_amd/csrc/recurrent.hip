@@ -2,8 +2,8 @@
 // float in the cache's state tensors: a gated linear recurrence whose forget gate also weighs the write
 // (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
 // channel) never meet: each needs only its own value and what the token brings per key channel (gates, keys,
-// queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns: lane (g, c) keeps rows
-// g, g + 4, g + 8, ... of column c in registers, the four lanes of a column add their parts of a dot product
+// queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns: lane (g, c) keeps a quarter of the
+// rows of column c in registers, the four lanes of a column add their parts of a dot product
 // with two cross-lane steps, and nothing waits for another wavefront.  What a token brings per key channel is
 // computed by the wavefront into its own piece of shared memory, from inputs it loaded one token ahead.  The
 // results go out unnormalised in float; a second kernel takes the root mean square over each head's value
@@ -17,9 +17,14 @@ __device__ __forceinline__ float blm_silu(float z) { return z / (1.0f + expf(-z)
 __device__ __forceinline__ float blm_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
 #define SCAN_COLS 16      // columns of the state per wavefront
-#define SCAN_GROUPS 4     // lanes per column; lane (g, c) holds rows g, g + 4, ...
+#define SCAN_GROUPS 4     // lanes per column; lane (g, c) holds rows g * ROWS .. g * ROWS + ROWS - 1
 #define SCAN_WAVES 4
 #define SCAN_MAX_DK 256
+// A vector per key channel in shared memory: channel i at i + 4 * (i / ROWS), so that the four groups' 16-byte
+// reads (each group's lanes read one address) fall on different banks; channels from dk up to 4 * ROWS hold zeros.
+#define SCAN_VEC (SCAN_MAX_DK + 4 * SCAN_GROUPS)
+template <int ROWS>
+__device__ __forceinline__ int scan_place(int i) { return i + 4 * (i / ROWS); }
 
 // ---------------------------------------------------------------------------------------
 // HGRN2.  proj [T][ld]: q at column 0 (H*dk), forget-gate logits at H*dk (H*dk), values at 2*H*dk (H*dv).
@@ -32,7 +37,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
                       const float* __restrict__ low, float* __restrict__ state, float* __restrict__ o_raw,
                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv,
                       int col_groups, long long n_items) {
-  __shared__ float sm[SCAN_WAVES][2][2 * SCAN_MAX_DK];     // per wavefront, two tokens: [f | q]
+  __shared__ __attribute__((aligned(16))) float sm[SCAN_WAVES][2][2 * SCAN_VEC];     // per wavefront, two tokens: [f | q]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
   if (item >= n_items) return;
@@ -48,9 +53,10 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   float S[ROWS];
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
-    const int i = r * SCAN_GROUPS + g;
+    const int i = g * ROWS + r;
     S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
   }
+  const int dkp = ROWS * SCAN_GROUPS;      // dk rounded up; the channels between stay zero
   // per key channel (lane l computes channels l, l + 64, ...): constants, and the token's raw inputs one ahead
   constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
   float lo[PER], fb[PER], raw_f[PER], raw_q[PER];
@@ -79,22 +85,25 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int i = lane + k * BLM_WAVE;
-      if (i < dk) {
-        fq[i] = lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[k] + fb[k]);
-        fq[dk + i] = blm_silu(raw_q[k]);
+      if (k * BLM_WAVE < dkp && i < dkp) {
+        fq[scan_place<ROWS>(i)] = i < dk ? lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[k] + fb[k]) : 0.f;
+        fq[SCAN_VEC + scan_place<ROWS>(i)] = i < dk ? blm_silu(raw_q[k]) : 0.f;
       }
     }
     const float v = v_next;
     if (t + 1 < t1) load_raw(t + 1, v_next);
     __builtin_amdgcn_wave_barrier();      // the piece of shared memory is the wavefront's own: reads follow writes in order
     float o = 0.f;
+    const float* fg = fq + g * (ROWS + 4);
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int i = r * SCAN_GROUPS + g;
-      if (i < dk) {
-        const float f = fq[i];
-        S[r] = fmaf(f, S[r], (1.f - f) * v);
-        o = fmaf(S[r], fq[dk + i], o);
+    for (int r = 0; r < ROWS; r += 4) {
+      const float4 f4 = *reinterpret_cast<const float4*>(fg + r);
+      const float4 q4 = *reinterpret_cast<const float4*>(fg + SCAN_VEC + r);
+      const float f[4] = {f4.x, f4.y, f4.z, f4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[r + e] = fmaf(f[e], S[r + e] - v, v);       // f S + (1 - f) v
+        o = fmaf(S[r + e], q[e], o);
       }
     }
     o = rows_sum(o);
@@ -104,7 +113,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   if (own) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      const int i = r * SCAN_GROUPS + g;
+      const int i = g * ROWS + r;
       if (i < dk) S_g[(size_t)i * dv + col] = S[r];
     }
   }
@@ -293,7 +302,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
                       const TA* __restrict__ decay_in, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
                       float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
                       const int* __restrict__ seq_slots, int H, int G, int dk, int dv, int col_groups, long long n_items) {
-  __shared__ float sm[SCAN_WAVES][2][3 * SCAN_MAX_DK];     // per wavefront, two tokens: [decay | k | q]
+  __shared__ __attribute__((aligned(16))) float sm[SCAN_WAVES][2][3 * SCAN_VEC];     // per wavefront, two tokens: [decay | k | q]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
   if (item >= n_items) return;
@@ -310,9 +319,10 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   float S[ROWS];
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
-    const int i = r * SCAN_GROUPS + g;
+    const int i = g * ROWS + r;
     S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
   }
+  const int dkp = ROWS * SCAN_GROUPS;
   constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
   const float rate = expf(a_log[h]);
   float bias[PER], raw_d[PER], raw_k[PER], raw_q[PER];
@@ -342,32 +352,40 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int i = lane + k * BLM_WAVE;
-      if (i < dk) {
-        buf[i] = expf(-rate * blm_softplus(raw_d[k] + bias[k]));
-        buf[dk + i] = raw_k[k];
-        buf[2 * dk + i] = raw_q[k];
+      if (k * BLM_WAVE < dkp && i < dkp) {
+        const int at = scan_place<ROWS>(i);
+        buf[at] = i < dk ? expf(-rate * blm_softplus(raw_d[k] + bias[k])) : 0.f;
+        buf[SCAN_VEC + at] = i < dk ? raw_k[k] : 0.f;
+        buf[2 * SCAN_VEC + at] = i < dk ? raw_q[k] : 0.f;
       }
     }
     const float v = v_next, beta = blm_sigmoid(bl_next);
     if (t + 1 < t1) load_raw(t + 1, v_next, bl_next);
     __builtin_amdgcn_wave_barrier();
+    const float* bg = buf + g * (ROWS + 4);
     float dot = 0.f;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int i = r * SCAN_GROUPS + g;
-      if (i < dk) {
-        S[r] *= buf[i];
-        dot = fmaf(S[r], buf[dk + i], dot);
+    for (int r = 0; r < ROWS; r += 4) {
+      const float4 d4 = *reinterpret_cast<const float4*>(bg + r);
+      const float4 k4 = *reinterpret_cast<const float4*>(bg + SCAN_VEC + r);
+      const float d[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[r + e] *= d[e];
+        dot = fmaf(S[r + e], kk[e], dot);
       }
     }
     const float u = beta * (v - rows_sum(dot));
     float o = 0.f;
 #pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-      const int i = r * SCAN_GROUPS + g;
-      if (i < dk) {
-        S[r] = fmaf(buf[dk + i], u, S[r]);
-        o = fmaf(S[r], buf[2 * dk + i], o);
+    for (int r = 0; r < ROWS; r += 4) {
+      const float4 k4 = *reinterpret_cast<const float4*>(bg + SCAN_VEC + r);
+      const float4 q4 = *reinterpret_cast<const float4*>(bg + 2 * SCAN_VEC + r);
+      const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[r + e] = fmaf(kk[e], u, S[r + e]);
+        o = fmaf(S[r + e], q[e], o);
       }
     }
     o = rows_sum(o);
@@ -377,7 +395,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   if (own) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
-      const int i = r * SCAN_GROUPS + g;
+      const int i = g * ROWS + r;
       if (i < dk) S_g[(size_t)i * dv + col] = S[r];
     }
   }
