@@ -144,20 +144,56 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The same for few rows (decoding): one wavefront per output column (h, n) streams that row of w once, its lanes
+// taking k = lane, lane + 64, ...; the rows' inputs come from the caches.  Up to HP_FEW rows.
+#define HP_FEW 16
+template <typename TI, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+    head_project_few_kernel(const TI* __restrict__ in, long long in_row, int in_head, const TW* __restrict__ w,
+                            TO* __restrict__ out, long long out_row, int out_head, int T, int H, int N, int K) {
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const long long col = (long long)blockIdx.x * 4 + wave;
+  if (col >= (long long)H * N) return;
+  const int h = (int)(col / N), n = (int)(col - (long long)h * N);
+  const TW* wr = w + ((size_t)h * N + n) * K;
+  const TI* a = in + (size_t)h * in_head;
+  float acc[HP_FEW];
+#pragma unroll
+  for (int t = 0; t < HP_FEW; ++t) acc[t] = 0.f;
+  for (int k = lane; k < K; k += BLM_WAVE) {
+    const float wv = to_float(wr[k]);
+#pragma unroll
+    for (int t = 0; t < HP_FEW; ++t)
+      if (t < T) acc[t] = fmaf(to_float(a[(size_t)t * in_row + k]), wv, acc[t]);
+  }
+#pragma unroll
+  for (int t = 0; t < HP_FEW; ++t) {
+    if (t < T) {
+      const float v = wave_sum(acc[t]);
+      if (lane == 0) out[(size_t)t * out_row + (size_t)h * out_head + n] = from_float<TO>(v);
+    }
+  }
+}
+
 extern "C" int blm_head_project(const void* in, int in_dtype, long long in_row, int in_head, const void* w, int w_dtype,
                                 void* out, int out_dtype, long long out_row, int out_head, int T, int H, int N, int K,
                                 hipStream_t stream) {
   BLM_REQUIRE(T > 0 && H > 0 && N > 0 && K > 0 && H <= 65535, "head_project: bad sizes T=%d H=%d N=%d K=%d", T, H, N, K);
   dim3 grid((T + HP_TILE - 1) / HP_TILE, (N + HP_TILE - 1) / HP_TILE, H), block(256);
   BLM_REQUIRE(grid.y <= 65535, "head_project: too many columns");
+  const unsigned few_blocks = (unsigned)(((long long)H * N + 3) / 4);
 #define BLM_HP(TI, TW, TO)                                                                                       \
-  hipLaunchKernelGGL((head_project_kernel<TI, TW, TO>), grid, block, 0, stream, (const TI*)in, in_row, in_head,  \
-                     (const TW*)w, (TO*)out, out_row, out_head, T, N, K)
-  if (in_dtype == BLM_F32 && w_dtype == BLM_F32 && out_dtype == BLM_F32) BLM_HP(float, float, float);
-  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) BLM_HP(bf16, bf16, float);
-  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) BLM_HP(float, bf16, bf16);
-  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) BLM_HP(bf16, bf16, bf16);
-  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) BLM_HP(float, bf16, float);
+  if (T <= HP_FEW)                                                                                               \
+    hipLaunchKernelGGL((head_project_few_kernel<TI, TW, TO>), dim3(few_blocks), block, 0, stream, (const TI*)in, \
+                       in_row, in_head, (const TW*)w, (TO*)out, out_row, out_head, T, H, N, K);                  \
+  else                                                                                                           \
+    hipLaunchKernelGGL((head_project_kernel<TI, TW, TO>), grid, block, 0, stream, (const TI*)in, in_row, in_head, \
+                       (const TW*)w, (TO*)out, out_row, out_head, T, N, K)
+  if (in_dtype == BLM_F32 && w_dtype == BLM_F32 && out_dtype == BLM_F32) { BLM_HP(float, float, float); }
+  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) { BLM_HP(bf16, bf16, float); }
+  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) { BLM_HP(float, bf16, bf16); }
+  else if (in_dtype == BLM_BF16 && w_dtype == BLM_BF16 && out_dtype == BLM_BF16) { BLM_HP(bf16, bf16, bf16); }
+  else if (in_dtype == BLM_F32 && w_dtype == BLM_BF16 && out_dtype == BLM_F32) { BLM_HP(float, bf16, float); }
   else return blm_fail("head_project: unsupported dtypes in=%d w=%d out=%d", in_dtype, w_dtype, out_dtype);
 #undef BLM_HP
   BLM_LAUNCH_CHECK("head_project");
@@ -517,11 +553,16 @@ __global__ void __launch_bounds__(LATM_WAVES* BLM_WAVE)
   }
 }
 
-// The pieces of a split run added up, one wavefront per column (a (token, head) pair): maxima in base 2.
-__global__ void __launch_bounds__(BLM_WAVE)
+// The pieces of a split run added up, one block per column (a (token, head) pair): maxima in base 2.  A piece
+// that saw nothing has sum 0, maximum -infinity and a result of zeros, and gets weight 0.
+#define LATM_MERGE_THREADS 256
+#define LATM_MAX_PIECES 64
+__global__ void __launch_bounds__(LATM_MERGE_THREADS)
     latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, float* __restrict__ olat,
                         const int* __restrict__ cu_seqlens, int H, int R, int tiles_per_seq, int n_splits) {
-  const int gcol = blockIdx.x, lane = threadIdx.x;
+  __shared__ float wgt[LATM_MAX_PIECES];
+  __shared__ float inv_sum;
+  const int gcol = blockIdx.x;
   const int per_seq = tiles_per_seq * 16;
   const int b = gcol / per_seq, idx = gcol - b * per_seq;
   const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
@@ -529,20 +570,21 @@ __global__ void __launch_bounds__(BLM_WAVE)
   const int tok = idx / H, head = idx - tok * H;
   float* orow = olat + ((size_t)(t_first + tok) * H + head) * R;
   const float* ml = part_ml + (size_t)gcol * n_splits * 2;
-  float M = -INFINITY;
-  for (int sp = 0; sp < n_splits; ++sp)
-    if (ml[sp * 2 + 1] != 0.f) M = fmaxf(M, ml[sp * 2]);
-  float L = 0.f;
-  for (int sp = 0; sp < n_splits; ++sp)
-    if (ml[sp * 2 + 1] != 0.f) L += ml[sp * 2 + 1] * __builtin_amdgcn_exp2f(ml[sp * 2] - M);
-  const float inv = 1.0f / L;
-  for (int d = lane; d < R; d += BLM_WAVE) {
+  if (threadIdx.x < BLM_WAVE) {          // n_splits <= 64: one lane per piece
+    const bool has = (int)threadIdx.x < n_splits;
+    const float ms = has ? ml[threadIdx.x * 2] : -INFINITY, ls = has ? ml[threadIdx.x * 2 + 1] : 0.f;
+    const float M = wave_max(ls != 0.f ? ms : -INFINITY);
+    const float w = ls != 0.f ? __builtin_amdgcn_exp2f(ms - M) : 0.f;
+    const float L = wave_sum(ls * w);
+    if (has) wgt[threadIdx.x] = w;
+    if (threadIdx.x == 0) inv_sum = 1.0f / L;
+  }
+  __syncthreads();
+  const float* po = part_o + (size_t)gcol * n_splits * R;
+  for (int d = threadIdx.x; d < R; d += LATM_MERGE_THREADS) {
     float acc = 0.f;
-    for (int sp = 0; sp < n_splits; ++sp) {
-      const float ls = ml[sp * 2 + 1];
-      if (ls != 0.f) acc = fmaf(part_o[((size_t)gcol * n_splits + sp) * R + d], __builtin_amdgcn_exp2f(ml[sp * 2] - M), acc);
-    }
-    orow[d] = acc * inv;
+    for (int sp = 0; sp < n_splits; ++sp) acc = fmaf(po[(size_t)sp * R + d], wgt[sp], acc);
+    orow[d] = acc * inv_sum;
   }
 }
 
@@ -565,8 +607,8 @@ extern "C" int blm_latent_attn_mfma(const void* q, float* olat, const int* cu_se
                                     float* part_o, float* part_ml, hipStream_t stream) {
   BLM_REQUIRE(B > 0 && max_new > 0 && H > 0, "latent_attn_mfma: bad sizes B=%d max_new=%d H=%d", B, max_new, H);
   BLM_REQUIRE(page_size == 64 && table_width > 0, "latent_attn_mfma: pages of 64 rows");
-  BLM_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml)),
-              "latent_attn_mfma: %d splits need their workspace", n_splits);
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= LATM_MAX_PIECES && (n_splits == 1 || (part_o && part_ml)),
+              "latent_attn_mfma: %d pieces (1 to %d, with their workspace)", n_splits, LATM_MAX_PIECES);
   const long long tiles = ((long long)max_new * H + 15) / 16;
   const long long waves = (long long)B * tiles;
   BLM_REQUIRE(waves < 2147483647LL, "latent_attn_mfma: too many tiles");
@@ -580,7 +622,7 @@ extern "C" int blm_latent_attn_mfma(const void* q, float* olat, const int* cu_se
                        B, H, (int)tiles, scale2, n_splits, part_o, part_ml);                                           \
     BLM_LAUNCH_CHECK("latent_attn_mfma");                                                                              \
     if (n_splits > 1) {                                                                                                \
-      hipLaunchKernelGGL(latent_merge_kernel, dim3((unsigned)(waves * 16)), dim3(BLM_WAVE), 0, stream, part_o, part_ml, \
+      hipLaunchKernelGGL(latent_merge_kernel, dim3((unsigned)(waves * 16)), dim3(LATM_MERGE_THREADS), 0, stream, part_o, part_ml, \
                          olat, cu_seqlens, H, R, (int)tiles, n_splits);                                                \
       BLM_LAUNCH_CHECK("latent_merge");                                                                                \
     }                                                                                                                  \

@@ -890,7 +890,7 @@ def head_project(x, in_head, w, out, out_head, K=None):
 
 
 _latent_scratch = {}
-LATENT_SCRATCH_FLOATS = 1 << 22
+LATENT_SCRATCH_FLOATS = 1 << 23
 
 
 def latent_attn_init(device):

@@ -20,16 +20,21 @@ __device__ __forceinline__ float blm_softplus(float z) { return fmaxf(z, 0.f) + 
 #define SCAN_GROUPS 4     // lanes per column; lane (g, c) holds rows g * ROWS .. g * ROWS + ROWS - 1
 #define SCAN_WAVES 4
 #define SCAN_MAX_DK 256
-// A vector per key channel in shared memory: channel i at i + 4 * (i / ROWS), so that the four groups' 16-byte
-// reads (each group's lanes read one address) fall on different banks; channels from dk up to 4 * ROWS hold zeros.
-#define SCAN_VEC (SCAN_MAX_DK + 4 * SCAN_GROUPS)
+// A vector per key channel in shared memory (4 * ROWS + 16 floats): channel i at i + 4 * (i / ROWS), so that the
+// four groups' 16-byte reads (each group's lanes read one address) fall on different banks; channels from dk up to
+// 4 * ROWS hold zeros.
 template <int ROWS>
 __device__ __forceinline__ int scan_place(int i) { return i + 4 * (i / ROWS); }
+
+#define SCAN_CHUNK 8      // tokens whose inputs a wavefront fetches and prepares at a time
 
 // ---------------------------------------------------------------------------------------
 // HGRN2.  proj [T][ld]: q at column 0 (H*dk), forget-gate logits at H*dk (H*dk), values at 2*H*dk (H*dv).
 //   f = low + (1 - low) * sigmoid(logit + bias);  S = diag(f) S + (1 - f) v^T;  o = S^T silu(q)
 // state [slots][H][dk][dv] float; o_raw [T][H*dv] float.
+// A wavefront takes its tokens eight at a time: the chunk's inputs were fetched into registers while the chunk
+// before ran (a trip to memory takes longer than a token's arithmetic), are turned into gates and activated
+// queries for all eight tokens at once, left in the wavefront's piece of shared memory, and walked in order.
 // ---------------------------------------------------------------------------------------
 template <typename TA, int ROWS>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
@@ -37,9 +42,9 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
                       const float* __restrict__ low, float* __restrict__ state, float* __restrict__ o_raw,
                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv,
                       int col_groups, long long n_items) {
-  __shared__ __attribute__((aligned(16))) float sm[SCAN_WAVES][2][2 * SCAN_VEC];     // per wavefront, two tokens: [f | q]
+  extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][f | q][vec], [chunk][16 values]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
-  const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
+  const long long item = (long long)blockIdx.x * (blockDim.x / BLM_WAVE) + wave;
   if (item >= n_items) return;
   const int cg = (int)(item % col_groups);
   const int h = (int)((item / col_groups) % H);
@@ -49,6 +54,10 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   if (slot < 0 || t1 <= t0) return;
   const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
   const bool own = col < dv;
+  constexpr int dkp = ROWS * SCAN_GROUPS;      // dk rounded up; the channels between stay zero
+  constexpr int vec = dkp + 16;
+  float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (2 * vec + SCAN_COLS);
+  float* v_sm = base + SCAN_CHUNK * 2 * vec;
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
   float S[ROWS];
 #pragma unroll
@@ -56,58 +65,73 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     const int i = g * ROWS + r;
     S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
   }
-  const int dkp = ROWS * SCAN_GROUPS;      // dk rounded up; the channels between stay zero
-  // per key channel (lane l computes channels l, l + 64, ...): constants, and the token's raw inputs one ahead
-  constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
-  float lo[PER], fb[PER], raw_f[PER], raw_q[PER];
+  // per key channel (lane l prepares channels l, l + 64, ...): constants, and a chunk's raw inputs
+  constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
+  float lo[PER], fb[PER], raw_f[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK];
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const int i = lane + k * BLM_WAVE;
     lo[k] = i < dk ? low[h * dk + i] : 0.f;
     fb[k] = i < dk ? f_bias[h * dk + i] : 0.f;
   }
-  auto load_raw = [&](int t, float& v) {
-    const TA* row = proj + (size_t)t * ld;
+  auto fetch = [&](int tc) {
 #pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int i = lane + k * BLM_WAVE;
-      if (i < dk) {
-        raw_f[k] = to_float(row[(size_t)H * dk + h * dk + i]);
-        raw_q[k] = to_float(row[h * dk + i]);
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tc + tt < t1) {
+        const TA* row = proj + (size_t)(tc + tt) * ld;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dk) {
+            raw_f[tt][k] = to_float(row[(size_t)H * dk + h * dk + i]);
+            raw_q[tt][k] = to_float(row[h * dk + i]);
+          }
+        }
+        v_in[tt] = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
       }
     }
-    v = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
   };
-  float v_next;
-  load_raw(t0, v_next);
-  for (int t = t0; t < t1; ++t) {
-    float* fq = sm[wave][(t - t0) & 1];
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += SCAN_CHUNK) {
+    const int n = min(SCAN_CHUNK, t1 - tc);
 #pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int i = lane + k * BLM_WAVE;
-      if (k * BLM_WAVE < dkp && i < dkp) {
-        fq[scan_place<ROWS>(i)] = i < dk ? lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[k] + fb[k]) : 0.f;
-        fq[SCAN_VEC + scan_place<ROWS>(i)] = i < dk ? blm_silu(raw_q[k]) : 0.f;
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tt < n) {
+        if (g == 0) v_sm[tt * SCAN_COLS + (lane & 15)] = v_in[tt];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dkp) {
+            const int at = scan_place<ROWS>(i);
+            base[(tt * 2) * vec + at] = i < dk ? lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[tt][k] + fb[k]) : 0.f;
+            base[(tt * 2 + 1) * vec + at] = i < dk ? blm_silu(raw_q[tt][k]) : 0.f;
+          }
+        }
       }
     }
-    const float v = v_next;
-    if (t + 1 < t1) load_raw(t + 1, v_next);
+    if (tc + SCAN_CHUNK < t1) fetch(tc + SCAN_CHUNK);     // the next chunk's inputs travel while this one runs
     __builtin_amdgcn_wave_barrier();      // the piece of shared memory is the wavefront's own: reads follow writes in order
-    float o = 0.f;
-    const float* fg = fq + g * (ROWS + 4);
+#pragma unroll 1
+    for (int tt = 0; tt < n; ++tt) {
+      {
+        const float* fg = base + (tt * 2) * vec + g * (ROWS + 4);
+        const float vv = v_sm[tt * SCAN_COLS + (lane & 15)];
+        float o = 0.f;
 #pragma unroll
-    for (int r = 0; r < ROWS; r += 4) {
-      const float4 f4 = *reinterpret_cast<const float4*>(fg + r);
-      const float4 q4 = *reinterpret_cast<const float4*>(fg + SCAN_VEC + r);
-      const float f[4] = {f4.x, f4.y, f4.z, f4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+        for (int r = 0; r < ROWS; r += 4) {
+          const float4 f4 = *reinterpret_cast<const float4*>(fg + r);
+          const float4 q4 = *reinterpret_cast<const float4*>(fg + vec + r);
+          const float f[4] = {f4.x, f4.y, f4.z, f4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        S[r + e] = fmaf(f[e], S[r + e] - v, v);       // f S + (1 - f) v
-        o = fmaf(S[r + e], q[e], o);
+          for (int e = 0; e < 4; ++e) {
+            S[r + e] = fmaf(f[e], S[r + e] - vv, vv);       // f S + (1 - f) v
+            o = fmaf(S[r + e], q[e], o);
+          }
+        }
+        o = rows_sum(o);
+        if (own && g == 0) o_raw[(size_t)(tc + tt) * H * dv + h * dv + col] = o;
       }
     }
-    o = rows_sum(o);
-    if (own && g == 0) o_raw[(size_t)t * H * dv + h * dv + col] = o;
     __builtin_amdgcn_wave_barrier();
   }
   if (own) {
@@ -152,6 +176,23 @@ static int launch_head_norm(const float* o_raw, const float* norm_w, const void*
   return 0;
 }
 
+// Wavefronts per block and shared memory of a scan whose wavefronts each keep `vectors` per-channel vectors for a
+// chunk of tokens: as many wavefronts (up to four) as fit the 64 KB a kernel gets without asking.
+struct ScanLaunch {
+  dim3 grid, block;
+  size_t smem;
+};
+static ScanLaunch scan_launch(int rows, int vectors, long long items) {
+  const size_t per_wave = (size_t)SCAN_CHUNK * (vectors * (rows * SCAN_GROUPS + 16) + (vectors - 1) * SCAN_COLS) * sizeof(float);
+  int waves = (int)((64 * 1024) / per_wave);
+  waves = waves > SCAN_WAVES ? SCAN_WAVES : (waves < 1 ? 1 : waves);
+  ScanLaunch sl;
+  sl.grid = dim3((unsigned)((items + waves - 1) / waves));
+  sl.block = dim3(waves * BLM_WAVE);
+  sl.smem = per_wave * waves;
+  return sl;
+}
+
 // rows per lane: the key channels dealt to four lanes, rounded up to what the kernels are built for
 #define BLM_SCAN_PICK(CALL)                   \
   do {                                        \
@@ -173,14 +214,13 @@ extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* 
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "hgrn2_scan: unsupported dtype %d", dtype);
   const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
   const long long items = (long long)B * H * col_groups;
-  const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
-  dim3 grid(blocks), block(SCAN_WAVES * BLM_WAVE);
 #define BLM_HG(ROWS)                                                                                                   \
+  const ScanLaunch sl = scan_launch(ROWS, 2, items);                                                                   \
   if (dtype == BLM_F32)                                                                                                \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), grid, block, 0, stream, (const float*)proj, ld, f_bias, low,  \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, f_bias, low, \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                             \
   else                                                                                                                 \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), grid, block, 0, stream, (const bf16*)proj, ld, f_bias, low,    \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, f_bias, low,   \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_HG);
 #undef BLM_HG
@@ -199,17 +239,21 @@ __global__ void conv_prepare_kernel(const TA* __restrict__ proj, int ld, const f
                                     const float* __restrict__ hist, float* __restrict__ out,
                                     const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
                                     const int* __restrict__ seq_slots, int C, int G, int dk) {
-  extern __shared__ float y[];
-  const int t = blockIdx.x;
+  // block (t, p): channels p * dk .. p * dk + dk - 1 of token t: a query or key head (p < 2 G), or as many values
+  __shared__ float red[17];
+  const int t = blockIdx.x, c0 = blockIdx.y * dk;
   const int b = token_seq[t];
   float* o = out + (size_t)t * C;
+  const int c_end = min(c0 + dk, C);
   if (b < 0) {
-    for (int c = threadIdx.x; c < C; c += blockDim.x) o[c] = 0.f;
+    for (int c = c0 + threadIdx.x; c < c_end; c += blockDim.x) o[c] = 0.f;
     return;
   }
   const int start = cu_seqlens[b], slot = seq_slots[b];
   const int off = t - start;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  const bool unit = c0 < 2 * G * dk;
+  float ss = 0.f;
+  for (int c = c0 + threadIdx.x; c < c_end; c += blockDim.x) {
     float a = 0.f;
     for (int k = 0; k < taps; ++k) {
       const int src = off - (taps - 1) + k;      // offset in the step of the input under tap k
@@ -218,21 +262,14 @@ __global__ void conv_prepare_kernel(const TA* __restrict__ proj, int ld, const f
       else x = slot >= 0 ? hist[((size_t)slot * (taps - 1) + (taps - 1 + src)) * C + c] : 0.f;
       a = fmaf(taps_w[(size_t)c * taps + k], x, a);
     }
-    y[c] = blm_silu(a);
+    a = blm_silu(a);
+    o[c] = a;
+    ss = fmaf(a, a, ss);
   }
-  __syncthreads();
-  const int n_qk = 2 * G * dk;
-  const float q_scale = 1.0f / sqrtf((float)dk);
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    float v = y[c];
-    if (c < n_qk) {
-      const float* head = y + (c / dk) * dk;
-      float ss = 0.f;
-      for (int i = 0; i < dk; ++i) ss = fmaf(head[i], head[i], ss);
-      v = v / sqrtf(ss + 1e-6f) * (c < G * dk ? q_scale : 1.f);
-    }
-    o[c] = v;
-  }
+  if (!unit) return;
+  ss = block_sum<true>(ss, red);
+  const float f = (c0 < G * dk ? 1.0f / sqrtf((float)dk) : 1.f) / sqrtf(ss + 1e-6f);
+  for (int c = c0 + threadIdx.x; c < c_end; c += blockDim.x) o[c] *= f;      // each thread rescales what it wrote
 }
 
 // The history after the step: the last taps-1 inputs of each sequence, taken from the step's rows and,
@@ -267,18 +304,20 @@ extern "C" int blm_conv_prepare(const void* proj, int dtype, int ld, const float
                                 int B, int C, int G, int dk, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && B > 0 && C > 0 && ld >= C, "conv_prepare: bad sizes T=%d B=%d C=%d ld=%d", T, B, C, ld);
   BLM_REQUIRE(taps >= 1 && taps <= BLM_MAX_TAPS, "conv_prepare: %d taps (1 to %d)", taps, BLM_MAX_TAPS);
-  BLM_REQUIRE(G >= 0 && dk >= 1 && 2 * G * dk <= C && (size_t)C * sizeof(float) <= 64 * 1024, "conv_prepare: bad head geometry");
+  BLM_REQUIRE(G >= 0 && dk >= 1 && 2 * G * dk <= C && true, "conv_prepare: bad head geometry");
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "conv_prepare: unsupported dtype %d", dtype);
-  const size_t smem = (size_t)C * sizeof(float);
   const unsigned ycols = (unsigned)((C + 255) / 256);
+  const unsigned pieces = (unsigned)((C + dk - 1) / dk);
+  const int threads = dk <= 64 ? 64 : (dk <= 128 ? 128 : 256);
+  BLM_REQUIRE(pieces <= 65535, "conv_prepare: too many heads");
   if (dtype == BLM_F32) {
-    hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(T), dim3(256), smem, stream, (const float*)proj, ld, taps_w, taps,
+    hipLaunchKernelGGL(conv_prepare_kernel<float>, dim3(T, pieces), dim3(threads), 0, stream, (const float*)proj, ld, taps_w, taps,
                        hist, out, token_seq, cu_seqlens, seq_slots, C, G, dk);
     if (taps > 1)
       hipLaunchKernelGGL(conv_history_kernel<float>, dim3(B, ycols), dim3(256), 0, stream, (const float*)proj, ld, taps, hist,
                          cu_seqlens, seq_slots, C);
   } else {
-    hipLaunchKernelGGL(conv_prepare_kernel<bf16>, dim3(T), dim3(256), smem, stream, (const bf16*)proj, ld, taps_w, taps,
+    hipLaunchKernelGGL(conv_prepare_kernel<bf16>, dim3(T, pieces), dim3(threads), 0, stream, (const bf16*)proj, ld, taps_w, taps,
                        hist, out, token_seq, cu_seqlens, seq_slots, C, G, dk);
     if (taps > 1)
       hipLaunchKernelGGL(conv_history_kernel<bf16>, dim3(B, ycols), dim3(256), 0, stream, (const bf16*)proj, ld, taps, hist,
@@ -302,9 +341,9 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
                       const TA* __restrict__ decay_in, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
                       float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
                       const int* __restrict__ seq_slots, int H, int G, int dk, int dv, int col_groups, long long n_items) {
-  __shared__ __attribute__((aligned(16))) float sm[SCAN_WAVES][2][3 * SCAN_VEC];     // per wavefront, two tokens: [decay | k | q]
+  extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][decay | k | q][vec], [chunk][16 values + beta]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
-  const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
+  const long long item = (long long)blockIdx.x * (blockDim.x / BLM_WAVE) + wave;
   if (item >= n_items) return;
   const int cg = (int)(item % col_groups);
   const int h = (int)((item / col_groups) % H);
@@ -315,6 +354,10 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
   const bool own = col < dv;
   const int kh = h / (H / G);
+  constexpr int dkp = ROWS * SCAN_GROUPS;
+  constexpr int vec = dkp + 16;
+  float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (3 * vec + 2 * SCAN_COLS);
+  float* v_sm = base + SCAN_CHUNK * 3 * vec;        // per token: 16 values, then beta
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
   float S[ROWS];
 #pragma unroll
@@ -322,74 +365,90 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     const int i = g * ROWS + r;
     S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
   }
-  const int dkp = ROWS * SCAN_GROUPS;
-  constexpr int PER = SCAN_MAX_DK / BLM_WAVE;
+  constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
   const float rate = expf(a_log[h]);
-  float bias[PER], raw_d[PER], raw_k[PER], raw_q[PER];
+  float bias[PER], raw_d[SCAN_CHUNK][PER], raw_k[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK], bl_in[SCAN_CHUNK];
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const int i = lane + k * BLM_WAVE;
     bias[k] = i < dk ? dt_bias[h * dk + i] : 0.f;
   }
-  auto load_raw = [&](int t, float& v, float& beta_logit) {
-    const float* row = qkv + (size_t)t * C;
+  auto fetch = [&](int tc) {
 #pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int i = lane + k * BLM_WAVE;
-      if (i < dk) {
-        raw_d[k] = to_float(decay_in[(size_t)t * H * dk + h * dk + i]);
-        raw_k[k] = row[(size_t)G * dk + kh * dk + i];
-        raw_q[k] = row[kh * dk + i];
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tc + tt < t1) {
+        const int t = tc + tt;
+        const float* row = qkv + (size_t)t * C;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dk) {
+            raw_d[tt][k] = to_float(decay_in[(size_t)t * H * dk + h * dk + i]);
+            raw_k[tt][k] = row[(size_t)G * dk + kh * dk + i];
+            raw_q[tt][k] = row[kh * dk + i];
+          }
+        }
+        v_in[tt] = own ? row[(size_t)2 * G * dk + h * dv + col] : 0.f;
+        bl_in[tt] = to_float(beta_src[(size_t)t * ld_beta + beta_col + h]);
       }
     }
-    v = own ? row[(size_t)2 * G * dk + h * dv + col] : 0.f;
-    beta_logit = to_float(beta_src[(size_t)t * ld_beta + beta_col + h]);
   };
-  float v_next, bl_next;
-  load_raw(t0, v_next, bl_next);
-  for (int t = t0; t < t1; ++t) {
-    float* buf = sm[wave][(t - t0) & 1];
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += SCAN_CHUNK) {
+    const int n = min(SCAN_CHUNK, t1 - tc);
 #pragma unroll
-    for (int k = 0; k < PER; ++k) {
-      const int i = lane + k * BLM_WAVE;
-      if (k * BLM_WAVE < dkp && i < dkp) {
-        const int at = scan_place<ROWS>(i);
-        buf[at] = i < dk ? expf(-rate * blm_softplus(raw_d[k] + bias[k])) : 0.f;
-        buf[SCAN_VEC + at] = i < dk ? raw_k[k] : 0.f;
-        buf[2 * SCAN_VEC + at] = i < dk ? raw_q[k] : 0.f;
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tt < n) {
+        if (g == 0) v_sm[tt * 2 * SCAN_COLS + (lane & 15)] = v_in[tt];
+        if (lane == 0) v_sm[tt * 2 * SCAN_COLS + SCAN_COLS] = blm_sigmoid(bl_in[tt]);
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dkp) {
+            const int at = scan_place<ROWS>(i);
+            base[(tt * 3) * vec + at] = i < dk ? expf(-rate * blm_softplus(raw_d[tt][k] + bias[k])) : 0.f;
+            base[(tt * 3 + 1) * vec + at] = i < dk ? raw_k[tt][k] : 0.f;
+            base[(tt * 3 + 2) * vec + at] = i < dk ? raw_q[tt][k] : 0.f;
+          }
+        }
       }
     }
-    const float v = v_next, beta = blm_sigmoid(bl_next);
-    if (t + 1 < t1) load_raw(t + 1, v_next, bl_next);
+    if (tc + SCAN_CHUNK < t1) fetch(tc + SCAN_CHUNK);     // the next chunk's inputs travel while this one runs
     __builtin_amdgcn_wave_barrier();
-    const float* bg = buf + g * (ROWS + 4);
-    float dot = 0.f;
+#pragma unroll 1
+    for (int tt = 0; tt < n; ++tt) {
+      {
+        const float* bg = base + (tt * 3) * vec + g * (ROWS + 4);
+        const float vv = v_sm[tt * 2 * SCAN_COLS + (lane & 15)], beta = v_sm[tt * 2 * SCAN_COLS + SCAN_COLS];
+        float dot = 0.f;
 #pragma unroll
-    for (int r = 0; r < ROWS; r += 4) {
-      const float4 d4 = *reinterpret_cast<const float4*>(bg + r);
-      const float4 k4 = *reinterpret_cast<const float4*>(bg + SCAN_VEC + r);
-      const float d[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w};
+        for (int r = 0; r < ROWS; r += 4) {
+          const float4 d4 = *reinterpret_cast<const float4*>(bg + r);
+          const float4 k4 = *reinterpret_cast<const float4*>(bg + vec + r);
+          const float d[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        S[r + e] *= d[e];
-        dot = fmaf(S[r + e], kk[e], dot);
+          for (int e = 0; e < 4; ++e) {
+            S[r + e] *= d[e];
+            dot = fmaf(S[r + e], kk[e], dot);
+          }
+        }
+        const float u = beta * (vv - rows_sum(dot));
+        float o = 0.f;
+#pragma unroll
+        for (int r = 0; r < ROWS; r += 4) {
+          const float4 k4 = *reinterpret_cast<const float4*>(bg + vec + r);
+          const float4 q4 = *reinterpret_cast<const float4*>(bg + 2 * vec + r);
+          const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            S[r + e] = fmaf(kk[e], u, S[r + e]);
+            o = fmaf(S[r + e], q[e], o);
+          }
+        }
+        o = rows_sum(o);
+        if (own && g == 0) o_raw[(size_t)(tc + tt) * H * dv + h * dv + col] = o;
       }
     }
-    const float u = beta * (v - rows_sum(dot));
-    float o = 0.f;
-#pragma unroll
-    for (int r = 0; r < ROWS; r += 4) {
-      const float4 k4 = *reinterpret_cast<const float4*>(bg + SCAN_VEC + r);
-      const float4 q4 = *reinterpret_cast<const float4*>(bg + 2 * SCAN_VEC + r);
-      const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        S[r + e] = fmaf(kk[e], u, S[r + e]);
-        o = fmaf(S[r + e], q[e], o);
-      }
-    }
-    o = rows_sum(o);
-    if (own && g == 0) o_raw[(size_t)t * H * dv + h * dv + col] = o;
     __builtin_amdgcn_wave_barrier();
   }
   if (own) {
@@ -412,15 +471,14 @@ extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "delta_scan: unsupported dtype %d", dtype);
   const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
   const long long items = (long long)B * H * col_groups;
-  const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
-  dim3 grid(blocks), block(SCAN_WAVES * BLM_WAVE);
 #define BLM_DS(ROWS)                                                                                                      \
+  const ScanLaunch sl = scan_launch(ROWS, 3, items);                                                                      \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), grid, block, 0, stream, qkv, C, (const float*)beta_src, ld_beta, \
+    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, (const float*)beta_src, ld_beta, \
                        beta_col, (const float*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,   \
                        dv, col_groups, items);                                                                            \
   else                                                                                                                    \
-    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), grid, block, 0, stream, qkv, C, (const bf16*)beta_src, ld_beta,   \
+    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, (const bf16*)beta_src, ld_beta, \
                        beta_col, (const bf16*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,    \
                        dv, col_groups, items)
   BLM_SCAN_PICK(BLM_DS);

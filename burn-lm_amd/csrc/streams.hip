@@ -95,7 +95,9 @@ static int launch_streams_norm(float* x, int S, const void* y, int n_planes, lon
                                const float* beta, void* out, const int* rows, int n_out, int D, float eps,
                                float out_scale, int write_x, const float* carry, float* stash, const int* token_seq,
                                const int* cu_seqlens, const int* seq_slots, const int* positions, hipStream_t stream) {
-  const int threads = D >= 1024 ? 512 : (D >= 256 ? 256 : 128);
+  // few rows (decoding): a row's loads are what the kernel waits for, so as many threads as the row has pairs of lanes
+  const int wide = ((D / 2 + BLM_WAVE - 1) / BLM_WAVE) * BLM_WAVE;
+  const int threads = n_out <= 512 ? (wide < 128 ? 128 : (wide > 1024 ? 1024 : wide)) : (D >= 1024 ? 512 : (D >= 256 ? 256 : 128));
   hipLaunchKernelGGL((streams_norm_kernel<TD, TO>), dim3(n_out), dim3(threads), (size_t)D * sizeof(float), stream, x, S,
                      (const TD*)y, n_planes, (size_t)plane_stride, scale_y, mix, outw, readw, gamma, beta, (TO*)out, rows, D,
                      eps, out_scale, write_x, carry, stash, token_seq, cu_seqlens, seq_slots, positions);

@@ -16,7 +16,7 @@ import torch
 from .base import KVNeed, Mixer, TensorSpec
 
 DECODE_BLOCKS_PER_UNIT = 2     # blocks of four (token, head) wavefronts the split decode aims for per compute unit
-MFMA_MAX_PIECES = 32           # most pieces the matrix-core decode cuts a sequence's pages into
+MFMA_MAX_PIECES = 64           # most pieces the matrix-core decode cuts a sequence's pages into
 
 
 class LatentAttention(Mixer):
@@ -102,8 +102,9 @@ class LatentAttention(Mixer):
             if step.max_new == 1:
                 waves = step.n_seqs * ((H + 15) // 16)
                 pages = (step.max_len_after + 63) // 64
-                # a wavefront for every vector unit of the chip, at least two pages to a piece
-                n_splits = max(1, min(pages // 2, (4 * rt.compute_units) // waves, MFMA_MAX_PIECES,
+                # up to a wavefront for every vector unit of the chip: a wavefront waits out a page's trip from memory
+                # with nothing else to do, so short pieces are what shortens the step
+                n_splits = max(1, min(pages, (4 * rt.compute_units) // waves, MFMA_MAX_PIECES,
                                       ops.latent_attn_mfma_max_splits(step.n_seqs, 1, H, R)))
             return ops.latent_attn_mfma(qabs, olat, view.k, view.v, step, view.block_table(step), view.page_size, H, R,
                                         dr, self.scale, n_splits)
