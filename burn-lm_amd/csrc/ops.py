@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 28
+ABI_VERSION = 29
 _lib = None
 _lock = threading.Lock()
 
@@ -41,13 +41,13 @@ _SIGNATURES = {
                          ctypes.c_longlong, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_latent_attn": [_c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int,
                         _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
-    "blm_hgrn2_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p,
+    "blm_hgrn2_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p,
                        _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_conv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                          _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_delta_scan": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                       _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                       _c_int, _c_int, _c_int, _c_void_p],
+                       _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_add_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_int, _c_void_p, _c_int,
                         _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_rope_kv_write": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -981,14 +981,15 @@ def hgrn2_scan(proj, f_bias, low, norm_w, eps, state, o_raw, out, step, H, dk, d
     out [T, H * dv] in proj's dtype."""
     _gpu(proj, f_bias, low, norm_w, state, o_raw, out)
     _f32("o_raw", o_raw, proj.shape[0] * H * dv)
+    gates = torch.empty(proj.shape[0], 2 * H * dk, dtype=torch.float32, device=proj.device)
     _f32("f_bias", f_bias, H * dk); _f32("low", low, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
     _contig("out", out)
     if proj.stride(1) != 1 or out.dtype != proj.dtype or tuple(out.shape) != (proj.shape[0], H * dv) \
             or tuple(state.shape[1:]) != (H, dk, dv):
         raise KernelError("hgrn2_scan: shapes do not fit")
     _call("blm_hgrn2_scan", proj.data_ptr(), _code(proj), proj.stride(0), f_bias.data_ptr(), low.data_ptr(),
-          norm_w.data_ptr(), float(eps), state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
-          step.seq_slots.data_ptr(), proj.shape[0], step.n_seqs, H, dk, dv, _stream())
+          norm_w.data_ptr(), float(eps), state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(),
+          step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), proj.shape[0], step.n_seqs, H, dk, dv, _stream())
     return out
 
 
@@ -1016,6 +1017,7 @@ def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_
     _gpu(qkv, beta_src, decay_in, dt_bias, a_log, gate_in, norm_w, state, o_raw, out)
     T, C = qkv.shape
     _f32("o_raw", o_raw, T * H * dv)
+    gates = torch.empty(T, H * dk + H, dtype=torch.float32, device=qkv.device)
     _f32("qkv", qkv); _f32("dt_bias", dt_bias, H * dk); _f32("a_log", a_log, H); _f32("norm_w", norm_w, dv)
     _f32("state", state)
     _contig("decay_in", decay_in); _contig("gate_in", gate_in); _contig("out", out)
@@ -1026,6 +1028,6 @@ def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_
         raise KernelError("delta_scan: shapes do not fit")
     _call("blm_delta_scan", qkv.data_ptr(), C, beta_src.data_ptr(), _code(out), beta_src.stride(0), beta_col,
           decay_in.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(), gate_in.data_ptr(), norm_w.data_ptr(), float(eps),
-          state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T,
-          step.n_seqs, H, G, dk, dv, _stream())
+          state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
+          step.seq_slots.data_ptr(), T, step.n_seqs, H, G, dk, dv, _stream())
     return out

@@ -35,11 +35,28 @@ __device__ __forceinline__ int scan_place(int i) { return i + 4 * (i / ROWS); }
 // A wavefront takes its tokens eight at a time: the chunk's inputs were fetched into registers while the chunk
 // before ran (a trip to memory takes longer than a token's arithmetic), are turned into gates and activated
 // queries for all eight tokens at once, left in the wavefront's piece of shared memory, and walked in order.
+// (The gates themselves come from hgrn2_gates_kernel.)
 // ---------------------------------------------------------------------------------------
+// gates [T][2 * H*dk] float: f = low + (1 - low) * sigmoid(logit + bias), then silu(q): everything about a token that
+// does not depend on the state, for all tokens at once, so that the walk in order does no more than it must
+template <typename TA>
+__global__ void hgrn2_gates_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ f_bias,
+                                   const float* __restrict__ low, float* __restrict__ gates, long long n, int HK) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / HK;
+    const int c = (int)(e - t * HK);
+    const TA* row = proj + (size_t)t * ld;
+    const float lo = low[c];
+    gates[(size_t)t * 2 * HK + c] = lo + (1.f - lo) * blm_sigmoid(to_float(row[HK + c]) + f_bias[c]);
+    gates[(size_t)t * 2 * HK + HK + c] = blm_silu(to_float(row[c]));
+  }
+}
+
 template <typename TA, int ROWS>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
-    hgrn2_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ f_bias,
-                      const float* __restrict__ low, float* __restrict__ state, float* __restrict__ o_raw,
+    hgrn2_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates,
+                      float* __restrict__ state, float* __restrict__ o_raw,
                       const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv,
                       int col_groups, long long n_items) {
   extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][f | q][vec], [chunk][16 values]
@@ -67,24 +84,19 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   }
   // per key channel (lane l prepares channels l, l + 64, ...): constants, and a chunk's raw inputs
   constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
-  float lo[PER], fb[PER], raw_f[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const int i = lane + k * BLM_WAVE;
-    lo[k] = i < dk ? low[h * dk + i] : 0.f;
-    fb[k] = i < dk ? f_bias[h * dk + i] : 0.f;
-  }
+  float raw_f[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK];
   auto fetch = [&](int tc) {
 #pragma unroll
     for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
       if (tc + tt < t1) {
         const TA* row = proj + (size_t)(tc + tt) * ld;
+        const float* gr = gates + (size_t)(tc + tt) * 2 * H * dk;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
           const int i = lane + k * BLM_WAVE;
           if (i < dk) {
-            raw_f[tt][k] = to_float(row[(size_t)H * dk + h * dk + i]);
-            raw_q[tt][k] = to_float(row[h * dk + i]);
+            raw_f[tt][k] = gr[h * dk + i];
+            raw_q[tt][k] = gr[(size_t)H * dk + h * dk + i];
           }
         }
         v_in[tt] = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
@@ -103,8 +115,8 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
           const int i = lane + k * BLM_WAVE;
           if (i < dkp) {
             const int at = scan_place<ROWS>(i);
-            base[(tt * 2) * vec + at] = i < dk ? lo[k] + (1.f - lo[k]) * blm_sigmoid(raw_f[tt][k] + fb[k]) : 0.f;
-            base[(tt * 2 + 1) * vec + at] = i < dk ? blm_silu(raw_q[tt][k]) : 0.f;
+            base[(tt * 2) * vec + at] = i < dk ? raw_f[tt][k] : 0.f;
+            base[(tt * 2 + 1) * vec + at] = i < dk ? raw_q[tt][k] : 0.f;
           }
         }
       }
@@ -205,7 +217,7 @@ static ScanLaunch scan_launch(int rows, int vectors, long long items) {
   } while (0)
 
 extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* f_bias, const float* low,
-                              const float* norm_w, float eps, float* state, float* o_raw, void* out,
+                              const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
                               const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv,
                               hipStream_t stream) {
   BLM_REQUIRE(T > 0 && B > 0 && H > 0, "hgrn2_scan: bad sizes T=%d B=%d H=%d", T, B, H);
@@ -214,13 +226,22 @@ extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* 
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "hgrn2_scan: unsupported dtype %d", dtype);
   const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
   const long long items = (long long)B * H * col_groups;
+  {   // gates and activated queries of every token [T][2 * H*dk]
+    const long long n = (long long)T * H * dk;
+    const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    if (dtype == BLM_F32)
+      hipLaunchKernelGGL(hgrn2_gates_kernel<float>, dim3(gblocks), dim3(256), 0, stream, (const float*)proj, ld, f_bias, low, gates, n, H * dk);
+    else
+      hipLaunchKernelGGL(hgrn2_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)proj, ld, f_bias, low, gates, n, H * dk);
+    BLM_LAUNCH_CHECK("hgrn2_gates");
+  }
 #define BLM_HG(ROWS)                                                                                                   \
   const ScanLaunch sl = scan_launch(ROWS, 2, items);                                                                   \
   if (dtype == BLM_F32)                                                                                                \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, f_bias, low, \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                             \
   else                                                                                                                 \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, f_bias, low,   \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_HG);
 #undef BLM_HG
@@ -335,10 +356,26 @@ extern "C" int blm_conv_prepare(const void* proj, int dtype, int ld, const float
 // then out = o / sqrt(mean(o^2) + eps) * norm_w * sigmoid(gate_in[t][h*dv+j]) by head_norm_kernel.
 // beta_logit: column `beta_col` of rows of `ld_beta` elements; decay_in, gate_in: [T][H*dk], [T][H*dv].
 // ---------------------------------------------------------------------------------------
+// gates [T][H*dk + H] float: the decays, then beta = sigmoid(logit) per head: what does not depend on the state
+template <typename TA>
+__global__ void delta_gates_kernel(const TA* __restrict__ beta_src, int ld_beta, int beta_col,
+                                   const TA* __restrict__ decay_in, const float* __restrict__ dt_bias,
+                                   const float* __restrict__ a_log, float* __restrict__ gates, long long n, int H, int dk) {
+  const int HK = H * dk, per = HK + H;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / per;
+    const int c = (int)(e - t * per);
+    if (c < HK)
+      gates[e] = expf(-expf(a_log[c / dk]) * blm_softplus(to_float(decay_in[(size_t)t * HK + c]) + dt_bias[c]));
+    else
+      gates[e] = blm_sigmoid(to_float(beta_src[(size_t)t * ld_beta + beta_col + (c - HK)]));
+  }
+}
+
 template <typename TA, int ROWS>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
-    delta_scan_kernel(const float* __restrict__ qkv, int C, const TA* __restrict__ beta_src, int ld_beta, int beta_col,
-                      const TA* __restrict__ decay_in, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+    delta_scan_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ gates,
                       float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
                       const int* __restrict__ seq_slots, int H, int G, int dk, int dv, int col_groups, long long n_items) {
   extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][decay | k | q][vec], [chunk][16 values + beta]
@@ -366,30 +403,25 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
   }
   constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
-  const float rate = expf(a_log[h]);
-  float bias[PER], raw_d[SCAN_CHUNK][PER], raw_k[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK], bl_in[SCAN_CHUNK];
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const int i = lane + k * BLM_WAVE;
-    bias[k] = i < dk ? dt_bias[h * dk + i] : 0.f;
-  }
+  float raw_d[SCAN_CHUNK][PER], raw_k[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK], bl_in[SCAN_CHUNK];
   auto fetch = [&](int tc) {
 #pragma unroll
     for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
       if (tc + tt < t1) {
         const int t = tc + tt;
         const float* row = qkv + (size_t)t * C;
+        const float* gr = gates + (size_t)t * (H * dk + H);
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
           const int i = lane + k * BLM_WAVE;
           if (i < dk) {
-            raw_d[tt][k] = to_float(decay_in[(size_t)t * H * dk + h * dk + i]);
+            raw_d[tt][k] = gr[h * dk + i];
             raw_k[tt][k] = row[(size_t)G * dk + kh * dk + i];
             raw_q[tt][k] = row[kh * dk + i];
           }
         }
         v_in[tt] = own ? row[(size_t)2 * G * dk + h * dv + col] : 0.f;
-        bl_in[tt] = to_float(beta_src[(size_t)t * ld_beta + beta_col + h]);
+        bl_in[tt] = gr[H * dk + h];
       }
     }
   };
@@ -400,13 +432,13 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
       if (tt < n) {
         if (g == 0) v_sm[tt * 2 * SCAN_COLS + (lane & 15)] = v_in[tt];
-        if (lane == 0) v_sm[tt * 2 * SCAN_COLS + SCAN_COLS] = blm_sigmoid(bl_in[tt]);
+        if (lane == 0) v_sm[tt * 2 * SCAN_COLS + SCAN_COLS] = bl_in[tt];
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
           const int i = lane + k * BLM_WAVE;
           if (i < dkp) {
             const int at = scan_place<ROWS>(i);
-            base[(tt * 3) * vec + at] = i < dk ? expf(-rate * blm_softplus(raw_d[tt][k] + bias[k])) : 0.f;
+            base[(tt * 3) * vec + at] = i < dk ? raw_d[tt][k] : 0.f;
             base[(tt * 3 + 1) * vec + at] = i < dk ? raw_k[tt][k] : 0.f;
             base[(tt * 3 + 2) * vec + at] = i < dk ? raw_q[tt][k] : 0.f;
           }
@@ -462,7 +494,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
 
 extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int dtype, int ld_beta, int beta_col,
                               const void* decay_in, const float* dt_bias, const float* a_log, const void* gate_in,
-                              const float* norm_w, float eps, float* state, float* o_raw, void* out,
+                              const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
                               const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int G, int dk, int dv,
                               hipStream_t stream) {
   BLM_REQUIRE(T > 0 && B > 0 && H > 0 && G > 0 && H % G == 0, "delta_scan: bad sizes T=%d B=%d H=%d G=%d", T, B, H, G);
@@ -471,16 +503,25 @@ extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "delta_scan: unsupported dtype %d", dtype);
   const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
   const long long items = (long long)B * H * col_groups;
+  {   // decays and write strengths of every token [T][H*dk + H]
+    const long long n = (long long)T * (H * dk + H);
+    const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    if (dtype == BLM_F32)
+      hipLaunchKernelGGL(delta_gates_kernel<float>, dim3(gblocks), dim3(256), 0, stream, (const float*)beta_src, ld_beta, beta_col,
+                         (const float*)decay_in, dt_bias, a_log, gates, n, H, dk);
+    else
+      hipLaunchKernelGGL(delta_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)beta_src, ld_beta, beta_col,
+                         (const bf16*)decay_in, dt_bias, a_log, gates, n, H, dk);
+    BLM_LAUNCH_CHECK("delta_gates");
+  }
 #define BLM_DS(ROWS)                                                                                                      \
   const ScanLaunch sl = scan_launch(ROWS, 3, items);                                                                      \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, (const float*)beta_src, ld_beta, \
-                       beta_col, (const float*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,   \
-                       dv, col_groups, items);                                                                            \
+    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw, \
+                       cu_seqlens, seq_slots, H, G, dk, dv, col_groups, items);                                           \
   else                                                                                                                    \
-    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, (const bf16*)beta_src, ld_beta, \
-                       beta_col, (const bf16*)decay_in, dt_bias, a_log, state, o_raw, cu_seqlens, seq_slots, H, G, dk,    \
-                       dv, col_groups, items)
+    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw,  \
+                       cu_seqlens, seq_slots, H, G, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_DS);
 #undef BLM_DS
   BLM_LAUNCH_CHECK("delta_scan");
