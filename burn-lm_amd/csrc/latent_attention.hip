@@ -589,7 +589,9 @@ __global__ void __launch_bounds__(LATM_MERGE_THREADS)
 }
 
 // the sizes the matrix-core form is built for (latent lanes, turned key lanes)
-#define BLM_LATM_SIZES(X) X(512, 64) X(256, 64) X(256, 32) X(128, 64) X(128, 32) X(64, 32) X(64, 16) X(32, 16)
+#define BLM_LATM_SIZES(X)                                                                                    \
+  X(512, 64) X(512, 32) X(384, 64) X(256, 64) X(256, 32) X(192, 64) X(192, 32) X(160, 32) X(128, 64) X(128, 32) \
+  X(128, 16) X(96, 32) X(96, 16) X(64, 64) X(64, 32) X(64, 16) X(48, 16) X(32, 16) X(32, 8)
 
 extern "C" int blm_latent_attn_mfma_supported(int R, int Dr) {
 #define BLM_LATM_HAS(r, d) if (R == r && Dr == d) return 1;

@@ -21,10 +21,10 @@ TOL = {"float32": 2e-5, "bfloat16": 8e-2}
 
 
 # ---- configurations and weights of the tests --------------------------------------------------
-def latent(heads=3, dim=8, rot_dim=8, vdim=12, kv_rank=24, base=10000.0, ff=80):
+def latent(heads=3, dim=8, rot_dim=8, vdim=12, kv_rank=24, base=10000.0, ff=80, turning=None):
     return dict(type="latent_attention",
                 mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
-                           rot=dict(base=base, dims=rot_dim), scale=1.0 / math.sqrt(dim + rot_dim)),
+                           rot=dict(base=base, dims=turning or rot_dim), scale=1.0 / math.sqrt(dim + rot_dim)),
                 mlp=None if ff is None else dict(kind="dense", ff=ff))
 
 
@@ -237,9 +237,10 @@ def whole(eng, toks):
 @pytest.mark.parametrize("layer", [latent(ff=None), hgrn(ff=None), delta(ff=None), delta(heads=2, kv_heads=2, conv=1, ff=None),
                                    latent(heads=5, dim=4, rot_dim=12, vdim=4, kv_rank=12, ff=40),
                                    latent(heads=5, dim=8, rot_dim=16, vdim=8, kv_rank=64, ff=None),
-                                   latent(heads=20, dim=8, rot_dim=32, vdim=4, kv_rank=64, ff=None)],
+                                   latent(heads=20, dim=8, rot_dim=32, vdim=4, kv_rank=64, ff=None),
+                                   latent(heads=4, dim=8, rot_dim=16, vdim=8, kv_rank=32, ff=None, turning=8, base=300.0)],
                          ids=["latent", "hgrn2", "delta", "delta_one_tap", "latent_with_ff", "latent_matrix_core_sizes",
-                              "latent_more_heads_than_a_tile"])
+                              "latent_more_heads_than_a_tile", "latent_some_lanes_do_not_turn"])
 def test_every_mixer_alone(tmp_path, layer, dtype):
     cfg = config([layer], streams=2)
     w = make_weights(cfg, 3)
