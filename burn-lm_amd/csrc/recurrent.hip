@@ -2,9 +2,9 @@
 // float in the cache's state tensors: a gated linear recurrence whose forget gate also weighs the write
 // (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
 // channel) never meet: each needs only its own value and what the token brings per key channel (gates, keys,
-// queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns: lane (g, c) keeps a quarter of the
-// rows of column c in registers, the four lanes of a column add their parts of a dot product
-// with two cross-lane steps, and nothing waits for another wavefront.  What a token brings per key channel is
+// queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns (or 4): the 4 (or 16) lanes of a
+// column each keep a share of its rows in registers and add their parts of a dot product with a few cross-lane
+// steps, and nothing waits for another wavefront.  What a token brings per key channel is
 // computed by the wavefront into its own piece of shared memory, from inputs it loaded one token ahead.  The
 // results go out unnormalised in float; a second kernel takes the root mean square over each head's value
 // lanes, the weight and (delta rule) the output gate.  The same kernels serve prompts and decoding.
@@ -16,15 +16,28 @@ __device__ __forceinline__ float blm_sigmoid(float z) { return 1.0f / (1.0f + ex
 __device__ __forceinline__ float blm_silu(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float blm_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-#define SCAN_COLS 16      // columns of the state per wavefront
-#define SCAN_GROUPS 4     // lanes per column; lane (g, c) holds rows g * ROWS .. g * ROWS + ROWS - 1
+// Two shapes of a wavefront (LPC lanes per column, 64 / LPC columns; lane group g holds rows g * ROWS .. + ROWS - 1):
+// 4 lanes per column for steps of few tokens per sequence (decoding): 16 neighbouring columns make the state's
+// rows come and go in 64-byte pieces, which is what such a step waits for;  16 lanes per column for prompts: a
+// token then costs a lane a quarter of the dependent instructions, which is what a long walk in order waits for.
+#define SCAN_COLS 16      // most columns of the state per wavefront
 #define SCAN_WAVES 4
 #define SCAN_MAX_DK 256
-// A vector per key channel in shared memory (4 * ROWS + 16 floats): channel i at i + 4 * (i / ROWS), so that the
-// four groups' 16-byte reads (each group's lanes read one address) fall on different banks; channels from dk up to
-// 4 * ROWS hold zeros.
+// A vector per key channel in shared memory (LPC * (ROWS + 4) floats): channel i at i + 4 * (i / ROWS), so that the
+// groups' 16-byte reads (each group's lanes read one address) fall on different banks; channels from dk up to
+// LPC * ROWS hold zeros.
 template <int ROWS>
 __device__ __forceinline__ int scan_place(int i) { return i + 4 * (i / ROWS); }
+// sum over the lanes of a column: 4 lanes a row of 16 apart, or the 16 lanes of a row
+template <int LPC>
+__device__ __forceinline__ float column_sum(float v) {
+  if (LPC == 4) return rows_sum(v);
+  v += blm_dpp<BLM_DPP_XOR1>(v);
+  v += blm_dpp<BLM_DPP_XOR2>(v);
+  v += blm_dpp<BLM_DPP_HALF_MIRROR>(v);
+  v += blm_dpp<BLM_DPP_MIRROR>(v);
+  return v;
+}
 
 #define SCAN_CHUNK 8      // tokens whose inputs a wavefront fetches and prepares at a time
 
@@ -53,7 +66,7 @@ __global__ void hgrn2_gates_kernel(const TA* __restrict__ proj, int ld, const fl
   }
 }
 
-template <typename TA, int ROWS>
+template <typename TA, int ROWS, int LPC>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     hgrn2_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates,
                       float* __restrict__ state, float* __restrict__ o_raw,
@@ -69,10 +82,12 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   const int slot = seq_slots[b];
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
   if (slot < 0 || t1 <= t0) return;
-  const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
+  constexpr int COLS = BLM_WAVE / LPC;
+  const int g = LPC == 4 ? lane >> 4 : lane & 15, cl = LPC == 4 ? lane & 15 : lane >> 4;
+  const int col = cg * COLS + cl;
   const bool own = col < dv;
-  constexpr int dkp = ROWS * SCAN_GROUPS;      // dk rounded up; the channels between stay zero
-  constexpr int vec = dkp + 16;
+  constexpr int dkp = ROWS * LPC;      // dk rounded up; the channels between stay zero
+  constexpr int vec = LPC * (ROWS + 4);
   float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (2 * vec + SCAN_COLS);
   float* v_sm = base + SCAN_CHUNK * 2 * vec;
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
@@ -109,7 +124,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
 #pragma unroll
     for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
       if (tt < n) {
-        if (g == 0) v_sm[tt * SCAN_COLS + (lane & 15)] = v_in[tt];
+        if (g == 0) v_sm[tt * SCAN_COLS + cl] = v_in[tt];
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
           const int i = lane + k * BLM_WAVE;
@@ -127,7 +142,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     for (int tt = 0; tt < n; ++tt) {
       {
         const float* fg = base + (tt * 2) * vec + g * (ROWS + 4);
-        const float vv = v_sm[tt * SCAN_COLS + (lane & 15)];
+        const float vv = v_sm[tt * SCAN_COLS + cl];
         float o = 0.f;
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
@@ -140,7 +155,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
             o = fmaf(S[r + e], q[e], o);
           }
         }
-        o = rows_sum(o);
+        o = column_sum<LPC>(o);
         if (own && g == 0) o_raw[(size_t)(tc + tt) * H * dv + h * dv + col] = o;
       }
     }
@@ -194,8 +209,8 @@ struct ScanLaunch {
   dim3 grid, block;
   size_t smem;
 };
-static ScanLaunch scan_launch(int rows, int vectors, long long items) {
-  const size_t per_wave = (size_t)SCAN_CHUNK * (vectors * (rows * SCAN_GROUPS + 16) + (vectors - 1) * SCAN_COLS) * sizeof(float);
+static ScanLaunch scan_launch(int rows, int lpc, int vectors, long long items) {
+  const size_t per_wave = (size_t)SCAN_CHUNK * (vectors * lpc * (rows + 4) + (vectors - 1) * SCAN_COLS) * sizeof(float);
   int waves = (int)((64 * 1024) / per_wave);
   waves = waves > SCAN_WAVES ? SCAN_WAVES : (waves < 1 ? 1 : waves);
   ScanLaunch sl;
@@ -205,15 +220,23 @@ static ScanLaunch scan_launch(int rows, int vectors, long long items) {
   return sl;
 }
 
-// rows per lane: the key channels dealt to four lanes, rounded up to what the kernels are built for
-#define BLM_SCAN_PICK(CALL)                   \
-  do {                                        \
-    const int rows = (dk + 3) / 4;            \
-    if (rows <= 4) { CALL(4); }               \
-    else if (rows <= 8) { CALL(8); }          \
-    else if (rows <= 16) { CALL(16); }        \
-    else if (rows <= 32) { CALL(32); }        \
-    else { CALL(64); }                        \
+// rows per lane: the key channels dealt to a column's lanes, rounded up to what the kernels are built for; 16 lanes
+// per column where the sequences bring many tokens each (see above)
+#define BLM_SCAN_PICK(CALL)                                  \
+  do {                                                       \
+    if (T > 4 * B) {                                         \
+      const int rows = (dk + 15) / 16;                       \
+      if (rows <= 4) { CALL(4, 16); }                        \
+      else if (rows <= 8) { CALL(8, 16); }                   \
+      else { CALL(16, 16); }                                 \
+    } else {                                                 \
+      const int rows = (dk + 3) / 4;                         \
+      if (rows <= 4) { CALL(4, 4); }                         \
+      else if (rows <= 8) { CALL(8, 4); }                    \
+      else if (rows <= 16) { CALL(16, 4); }                  \
+      else if (rows <= 32) { CALL(32, 4); }                  \
+      else { CALL(64, 4); }                                  \
+    }                                                        \
   } while (0)
 
 extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* f_bias, const float* low,
@@ -224,8 +247,6 @@ extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* 
   BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "hgrn2_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(ld >= 2 * H * dk + H * dv, "hgrn2_scan: rows of %d are too short", ld);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "hgrn2_scan: unsupported dtype %d", dtype);
-  const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
-  const long long items = (long long)B * H * col_groups;
   {   // gates and activated queries of every token [T][2 * H*dk]
     const long long n = (long long)T * H * dk;
     const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
@@ -235,13 +256,15 @@ extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* 
       hipLaunchKernelGGL(hgrn2_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)proj, ld, f_bias, low, gates, n, H * dk);
     BLM_LAUNCH_CHECK("hgrn2_gates");
   }
-#define BLM_HG(ROWS)                                                                                                   \
-  const ScanLaunch sl = scan_launch(ROWS, 2, items);                                                                   \
+#define BLM_HG(ROWS, LPC)                                                                                              \
+  const int col_groups = (dv + 64 / LPC - 1) / (64 / LPC);                                                             \
+  const long long items = (long long)B * H * col_groups;                                                               \
+  const ScanLaunch sl = scan_launch(ROWS, LPC, 2, items);                                                              \
   if (dtype == BLM_F32)                                                                                                \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<float, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                             \
   else                                                                                                                 \
-    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
+    hipLaunchKernelGGL((hgrn2_scan_kernel<bf16, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
                        state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_HG);
 #undef BLM_HG
@@ -373,7 +396,7 @@ __global__ void delta_gates_kernel(const TA* __restrict__ beta_src, int ld_beta,
   }
 }
 
-template <typename TA, int ROWS>
+template <typename TA, int ROWS, int LPC>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     delta_scan_kernel(const float* __restrict__ qkv, int C, const float* __restrict__ gates,
                       float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
@@ -388,11 +411,13 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   const int slot = seq_slots[b];
   const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
   if (slot < 0 || t1 <= t0) return;
-  const int g = lane >> 4, col = cg * SCAN_COLS + (lane & 15);
+  constexpr int COLS = BLM_WAVE / LPC;
+  const int g = LPC == 4 ? lane >> 4 : lane & 15, cl = LPC == 4 ? lane & 15 : lane >> 4;
+  const int col = cg * COLS + cl;
   const bool own = col < dv;
   const int kh = h / (H / G);
-  constexpr int dkp = ROWS * SCAN_GROUPS;
-  constexpr int vec = dkp + 16;
+  constexpr int dkp = ROWS * LPC;
+  constexpr int vec = LPC * (ROWS + 4);
   float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (3 * vec + 2 * SCAN_COLS);
   float* v_sm = base + SCAN_CHUNK * 3 * vec;        // per token: 16 values, then beta
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
@@ -431,7 +456,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
 #pragma unroll
     for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
       if (tt < n) {
-        if (g == 0) v_sm[tt * 2 * SCAN_COLS + (lane & 15)] = v_in[tt];
+        if (g == 0) v_sm[tt * 2 * SCAN_COLS + cl] = v_in[tt];
         if (lane == 0) v_sm[tt * 2 * SCAN_COLS + SCAN_COLS] = bl_in[tt];
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
@@ -451,7 +476,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     for (int tt = 0; tt < n; ++tt) {
       {
         const float* bg = base + (tt * 3) * vec + g * (ROWS + 4);
-        const float vv = v_sm[tt * 2 * SCAN_COLS + (lane & 15)], beta = v_sm[tt * 2 * SCAN_COLS + SCAN_COLS];
+        const float vv = v_sm[tt * 2 * SCAN_COLS + cl], beta = v_sm[tt * 2 * SCAN_COLS + SCAN_COLS];
         float dot = 0.f;
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
@@ -464,7 +489,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
             dot = fmaf(S[r + e], kk[e], dot);
           }
         }
-        const float u = beta * (vv - rows_sum(dot));
+        const float u = beta * (vv - column_sum<LPC>(dot));
         float o = 0.f;
 #pragma unroll
         for (int r = 0; r < ROWS; r += 4) {
@@ -477,7 +502,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
             o = fmaf(S[r + e], q[e], o);
           }
         }
-        o = rows_sum(o);
+        o = column_sum<LPC>(o);
         if (own && g == 0) o_raw[(size_t)(tc + tt) * H * dv + h * dv + col] = o;
       }
     }
@@ -501,8 +526,6 @@ extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int
   BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "delta_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(C >= 2 * G * dk + H * dv, "delta_scan: rows of %d are too short", C);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "delta_scan: unsupported dtype %d", dtype);
-  const int col_groups = (dv + SCAN_COLS - 1) / SCAN_COLS;
-  const long long items = (long long)B * H * col_groups;
   {   // decays and write strengths of every token [T][H*dk + H]
     const long long n = (long long)T * (H * dk + H);
     const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
@@ -514,13 +537,15 @@ extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int
                          (const bf16*)decay_in, dt_bias, a_log, gates, n, H, dk);
     BLM_LAUNCH_CHECK("delta_gates");
   }
-#define BLM_DS(ROWS)                                                                                                      \
-  const ScanLaunch sl = scan_launch(ROWS, 3, items);                                                                      \
+#define BLM_DS(ROWS, LPC)                                                                                                 \
+  const int col_groups = (dv + 64 / LPC - 1) / (64 / LPC);                                                                \
+  const long long items = (long long)B * H * col_groups;                                                                  \
+  const ScanLaunch sl = scan_launch(ROWS, LPC, 3, items);                                                                 \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw, \
+    hipLaunchKernelGGL((delta_scan_kernel<float, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw, \
                        cu_seqlens, seq_slots, H, G, dk, dv, col_groups, items);                                           \
   else                                                                                                                    \
-    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw,  \
+    hipLaunchKernelGGL((delta_scan_kernel<bf16, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, qkv, C, gates, state, o_raw,  \
                        cu_seqlens, seq_slots, H, G, dk, dv, col_groups, items)
   BLM_SCAN_PICK(BLM_DS);
 #undef BLM_DS
