@@ -90,7 +90,11 @@ def cmd_random(args):
     from ..weights.random_init import write_model_folder
     cfg = preset(args.preset)
     if args.layers:
-        cfg["num_hidden_layers"] = args.layers
+        if isinstance(cfg.get("layers"), list):      # a configuration that lists its layers: the first so many
+            cfg["layers"] = cfg["layers"][:args.layers]
+            cfg.pop("loop", None)
+        else:
+            cfg["num_hidden_layers"] = args.layers
     folder = os.path.join(models_dir(), args.name or args.preset)
     print(f"writing random weights (seed {args.seed}) for {args.preset} into {folder} ...")
     write_model_folder(folder, cfg, seed=args.seed)

@@ -109,9 +109,14 @@ def test_plan_follows_the_configuration():
 
 
 def test_presets_are_valid_configurations():
+    from burn_lm_amd import registry
+    import burn_lm_amd.models  # noqa: F401
     for name in presets():
-        c = LlamaConfig.from_dict(preset(name))
-        assert c.num_hidden_layers > 0
+        arch = registry.architecture_of(preset(name))       # every preset names a registered architecture ...
+        c = arch.read_config(preset(name))                  # ... and is a configuration it accepts
+        assert c.vocab_size > 0 and c.max_positions > 0
+        if arch.name == "LlamaForCausalLM":
+            assert c.num_hidden_layers > 0
     c = LlamaConfig.from_dict(preset("llama3.2-1b"))
     # crates/burn-lm-llama/src/nn/llama/base.rs:103-113
     assert (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads,
