@@ -243,16 +243,16 @@ class Cache:
             g.pool = PagePool(g.n_pages, _native=_core.NativePool(g.n_pages, handle=lib.blm_cache_pool(self._h, gi)))
             g.tables = _Tables(self, gi)
 
-    def bytes_read(self, length: int) -> int:
+    def bytes_read(self, length: int, with_state: bool = False) -> int:
         """Bytes of keys and values that one step reads for a sequence of `length` tokens: every
         place of the order reads its group's keys and values (a place that shares another's cache
-        reads them again), all of them or the last window."""
+        reads them again), all of them or the last window.  with_state: fixed-size state counts too."""
         total = 0
         for v in (c for v in self.views for c in (v if isinstance(v, tuple) else (v,))):
             if isinstance(v, KVView):
                 keys = min(length, v.need.window) if v.need.window > 0 else length
                 total += (v.need.n_kv_heads * v.need.head_dim + v.need.v_heads * v.need.v_dim) * keys * v.k.element_size()
-            elif isinstance(v, StateView):      # fixed-size state is read and written once a step
+            elif with_state and isinstance(v, StateView):      # fixed-size state is read and written once a step
                 total += 2 * v.tensor[0].numel() * v.tensor.element_size()
         return total
 

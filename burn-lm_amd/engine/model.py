@@ -91,7 +91,7 @@ class Model:
                     flops += sum(part.mixing_flops(p, n) for p, n in zip(pasts, news))
         cache_bytes = 0
         if cache is not None:
-            cache_bytes = sum(cache.bytes_read(p + n) for p, n in zip(pasts, news))
+            cache_bytes = sum(cache.bytes_read(p + n, with_state=True) for p, n in zip(pasts, news))
         return dict(weight_bytes=weight_bytes, cache_bytes=cache_bytes, flops=flops)
 
     def forward(self, step, cache):
