@@ -1,6 +1,6 @@
 // Recurrent mixers whose state is a matrix [key channels][value channels] per head and sequence, kept in
-// float in the cache's state tensors: a gated linear recurrence whose forget gate also weighs the write
-// (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
+// float in the cache's state tensors: a linear recurrence with one gate that shares a channel between its old state and
+// the new value (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
 // channel) never meet: each needs only its own value and what the token brings per key channel (gates, keys,
 // queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns (or 4): the 4 (or 16) lanes of a
 // column each keep a share of its rows in registers and add their parts of a dot product with a few cross-lane

@@ -1,4 +1,4 @@
-"""Gated delta rule with one decay per head and key channel.
+"""Delta-rule mixer whose state decays channel by channel (a decay for every key channel of every head).
 
 ``q = W_q x`` and ``k = W_k x`` (kv_heads x dim), ``v = W_v x`` (heads x vdim); each passes a short causal
 convolution per channel and SiLU; q and k become unit vectors per head (q also times dim^-1/2); head h reads

@@ -1,4 +1,5 @@
-"""HGRN2: a gated linear recurrence in which the forget gate also decides what is written.
+"""HGRN2: a linear recurrence over a matrix state per head with a single gate: what a channel keeps of its old
+state is `f`, and what it takes of the new value is `1 - f`.
 
 ``q = silu(W_q x)``, ``v = W_v x``, ``f = low + (1 - low) * sigmoid(W_f x + b_f)`` per head and key channel
 (``low`` a stored lower bound); per head ``S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T`` and ``o_t = S_t^T q_t``

@@ -97,7 +97,7 @@ def latent_attention(x, w, p, m, eps, start=0):
 
 
 def hgrn2(x, w, p, m, eps, state=None):
-    """Gated linear recurrence whose forget gate also weighs the write.  Returns (y, state)."""
+    """Linear recurrence with one gate f per channel: f of the old state, 1 - f of the new value.  Returns (y, state)."""
     T = x.shape[0]
     H, dk, dv = m["heads"], m["dim"], m["vdim"]
     q = silu(x @ w[p + "q"].T).reshape(T, H, dk)
