@@ -171,7 +171,8 @@ class Cache:
     of them for a block whose parts each keep something of their own (keys and values beside a
     state, two sets of keys and values); its view is then a tuple in the same order.
     reads_from[i] is the earlier place whose keys and values place i reads instead of keeping
-    its own (or None); both places then have one need each."""
+    its own (or None); where either place has several needs, the keys and values are those of its
+    (first) KVNeed, and the reading place's states stay its own."""
 
     def __init__(self, needs: Sequence, reads_from: Sequence[Optional[int]], max_tokens: int,
                  max_seqs: int, max_context: int, page_size: int = 64, dtype=torch.bfloat16,
@@ -189,9 +190,6 @@ class Cache:
         cells: List[Tuple] = []
         for i, need in enumerate(needs):
             if isinstance(need, (tuple, list)):
-                if reads_from[i] is not None:
-                    raise CacheError(f"place {i} of the layer order has several needs and keeps them all itself: "
-                                     f"it cannot read the cache of place {reads_from[i]}")
                 cells += [((i, j), n) for j, n in enumerate(need)]
             else:
                 cells.append(((i, None), need))
@@ -210,19 +208,31 @@ class Cache:
             self.groups.append(g)
             for plane, key in enumerate(keys):
                 cell_views[key] = KVView(g, gi, plane, store=True)
+
+        def kept_by(src):
+            """(cell, view) of the keys and values that place src keeps itself: its one need, or the first
+            KVNeed among several."""
+            for key, _ in cells:
+                if key[0] == src and isinstance(cell_views[key], KVView) and cell_views[key].store:
+                    return key, cell_views[key]
+            return None, None
+
         for key, need in cells:
             i = key[0]
             src = reads_from[i]
-            if src is not None:
-                sv = cell_views.get((src, None)) if 0 <= src < i else None
-                if reads_from[src] is not None or not isinstance(sv, KVView):
+            several = key[1] is not None
+            if src is not None and (isinstance(need, KVNeed) or not several):
+                # a place with one need reads the other's keys and values whatever it asks for itself; among several
+                # needs the KVNeed does, and the states stay the place's own
+                sk, sv = kept_by(src) if 0 <= src < i and reads_from[src] is None else (None, None)
+                if sv is None:
                     raise CacheError(f"place {i} of the layer order reads the cache of place {src}, which must be "
                                      f"an earlier place that keeps keys and values of its own")
                 if isinstance(need, KVNeed) and (need.n_kv_heads, need.head_dim, need.v_heads, need.v_dim) != \
                         (sv.need.n_kv_heads, sv.need.head_dim, sv.need.v_heads, sv.need.v_dim):
                     raise CacheError(f"place {i} cannot read the cache of place {src}: head counts or sizes differ")
                 g = self.groups[sv.group_index]
-                cell_views[key] = KVView(g, sv.group_index, g.places.index((src, None)), store=False)
+                cell_views[key] = KVView(g, sv.group_index, g.places.index(sk), store=False)
             elif isinstance(need, StateNeed):
                 t = torch.zeros(max_seqs, *need.shape, dtype=need.dtype, device=device)
                 self.state_tensors.append(t)

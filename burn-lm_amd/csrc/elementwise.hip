@@ -8,27 +8,28 @@
 // ---------------------------------------------------------------------------------------
 template <typename TW>
 __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ h, int D, int copies) {
+                                    float* __restrict__ h, int D, int copies, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   const TW* row = table + (size_t)id * D;
   float* out = h + (size_t)t * copies * D;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float v = to_float(row[d]);
+    const float v = to_float(row[d]) * scale;
     for (int c = 0; c < copies; ++c) out[(size_t)c * D + d] = v;
   }
 }
 
+// scale: every element is multiplied by it (1: the table's rows as they are).
 // copies: h is [T][copies][D] and every copy of a token's row is the same (residual arrangements with
 // several streams start from equal streams)
 extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* ids, float* h,
-                                int T, int D, int copies, hipStream_t stream) {
+                                int T, int D, int copies, float scale, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && D > 0 && copies >= 1, "embed_gather: bad sizes T=%d D=%d copies=%d", T, D, copies);
   dim3 grid(T), block(256);
   if (table_dtype == BLM_F32)
-    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, (const float*)table, ids, h, D, copies);
+    hipLaunchKernelGGL(embed_gather_kernel<float>, grid, block, 0, stream, (const float*)table, ids, h, D, copies, scale);
   else if (table_dtype == BLM_BF16)
-    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, h, D, copies);
+    hipLaunchKernelGGL(embed_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, h, D, copies, scale);
   else
     return blm_fail("embed_gather: unsupported table dtype %d", table_dtype);
   BLM_LAUNCH_CHECK("embed_gather");
@@ -42,7 +43,7 @@ extern "C" int blm_embed_gather(const void* table, int table_dtype, const int* i
 template <typename TW>
 __global__ void embed_gather_from_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
                                          const int* __restrict__ source_rows, const int* const* __restrict__ source,
-                                         float* __restrict__ h, int D, int V, int copies) {
+                                         float* __restrict__ h, int D, int V, int copies, float scale) {
   const int t = blockIdx.x;
   const int r = source_rows[t];
   const int id = r >= 0 ? (*source)[r] : ids[t];
@@ -53,13 +54,14 @@ __global__ void embed_gather_from_kernel(const TW* __restrict__ table, const int
   }
   const TW* row = table + (size_t)id * D;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    const float v = to_float(row[d]);
+    const float v = to_float(row[d]) * scale;
     for (int c = 0; c < copies; ++c) out[(size_t)c * D + d] = v;
   }
 }
 
 extern "C" int blm_embed_gather_from(const void* table, int table_dtype, const int* ids, const int* source_rows,
-                                     const void* source_cell, float* h, int T, int D, int V, int copies, hipStream_t stream) {
+                                     const void* source_cell, float* h, int T, int D, int V, int copies, float scale,
+                                     hipStream_t stream) {
   BLM_REQUIRE(T > 0 && D > 0 && V > 0 && copies >= 1, "embed_gather_from: bad sizes T=%d D=%d V=%d", T, D, V);
   BLM_REQUIRE(source_rows && source_cell && ((size_t)source_cell & 7) == 0,
               "embed_gather_from: needs the rows and an 8-byte aligned cell with the tokens' address");
@@ -67,10 +69,10 @@ extern "C" int blm_embed_gather_from(const void* table, int table_dtype, const i
   const int* const* cell = (const int* const*)source_cell;
   if (table_dtype == BLM_F32)
     hipLaunchKernelGGL(embed_gather_from_kernel<float>, grid, block, 0, stream, (const float*)table, ids, source_rows,
-                       cell, h, D, V, copies);
+                       cell, h, D, V, copies, scale);
   else if (table_dtype == BLM_BF16)
     hipLaunchKernelGGL(embed_gather_from_kernel<bf16>, grid, block, 0, stream, (const bf16*)table, ids, source_rows,
-                       cell, h, D, V, copies);
+                       cell, h, D, V, copies, scale);
   else
     return blm_fail("embed_gather_from: unsupported table dtype %d", table_dtype);
   BLM_LAUNCH_CHECK("embed_gather_from");

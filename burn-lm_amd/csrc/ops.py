@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 29
+ABI_VERSION = 30
 _lib = None
 _lock = threading.Lock()
 
@@ -22,9 +22,26 @@ class KernelError(RuntimeError):
 
 
 _SIGNATURES = {
-    "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_embed_gather": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_void_p],
     "blm_embed_gather_from": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
-                              _c_int, _c_void_p],
+                              _c_int, _c_float, _c_void_p],
+    "blm_input_conv": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p,
+                       _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_residual_add": [_c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int,
+                         _c_int, _c_void_p],
+    "blm_side_gate": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                      _c_int, _c_int, _c_void_p],
+    "blm_rms_scale": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
+    "blm_clamped_glu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void_p],
+    "blm_moe_route": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
+    "blm_moe_gate": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_gla_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_float, _c_void_p, _c_void_p,
+                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
+                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_sink_attn": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                      _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                      _c_void_p],
     "blm_streams_norm": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_void_p, _c_void_p,
                          _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_float,
                          _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
@@ -213,18 +230,19 @@ def _embed_shape(who, table, out_h):
     return out_h.shape[0], out_h.shape[-1], (out_h.shape[1] if out_h.dim() == 3 else 1)
 
 
-def embed_gather(table, ids, out_h):
-    """out_h[t, :] = table[ids[t], :] as float32 (out_h [T, copies, D]: every copy alike).  ids must already be
-    checked against the vocabulary."""
+def embed_gather(table, ids, out_h, scale=1.0):
+    """out_h[t, :] = table[ids[t], :] * scale as float32 (out_h [T, copies, D]: every copy alike).  ids must already
+    be checked against the vocabulary."""
     _gpu(table, ids, out_h)
     T, D, copies = _embed_shape("embed_gather", table, out_h)
     _i32("ids", ids, T)
     _contig("table", table); _contig("h", out_h)
-    _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, copies, _stream())
+    _call("blm_embed_gather", table.data_ptr(), _code(table), ids.data_ptr(), out_h.data_ptr(), T, D, copies, float(scale),
+          _stream())
     return out_h
 
 
-def embed_gather_from(table, ids, source_rows, source_cell, out_h):
+def embed_gather_from(table, ids, source_rows, source_cell, out_h, scale=1.0):
     """Like embed_gather, but row t's token is taken on the device where source_rows[t] >= 0: it is
     element source_rows[t] of the int32 array whose address stands in source_cell (an int64 tensor of
     one element on the device).  A token outside the vocabulary gives a row of NaN."""
@@ -236,7 +254,7 @@ def embed_gather_from(table, ids, source_rows, source_cell, out_h):
     if source_cell.dtype != torch.int64 or source_cell.numel() != 1:
         raise KernelError("embed_gather_from: the cell is one int64 on the device")
     _call("blm_embed_gather_from", table.data_ptr(), _code(table), ids.data_ptr(), source_rows.data_ptr(),
-          source_cell.data_ptr(), out_h.data_ptr(), T, D, table.shape[0], copies, _stream())
+          source_cell.data_ptr(), out_h.data_ptr(), T, D, table.shape[0], copies, float(scale), _stream())
     return out_h
 
 
@@ -1030,4 +1048,200 @@ def delta_scan(qkv, beta_src, beta_col, decay_in, dt_bias, a_log, gate_in, norm_
           decay_in.data_ptr(), dt_bias.data_ptr(), a_log.data_ptr(), gate_in.data_ptr(), norm_w.data_ptr(), float(eps),
           state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(),
           step.seq_slots.data_ptr(), T, step.n_seqs, H, G, dk, dv, _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# layers whose sublayers run side by side: input convolution, residual add, side input, clamped and routed gating
+def _planes(who, y, T, D):
+    """(planes, dtype code) of a sublayer's result: [T, D], or float32 planes [P, T, D]."""
+    _contig(who, y)
+    if y.dim() == 3:
+        if tuple(y.shape[1:]) != (T, D) or y.dtype != torch.float32:
+            raise KernelError(f"{who}: partial results must be float32 [planes, {T}, {D}], got {tuple(y.shape)}")
+        return y.shape[0], 0
+    if tuple(y.shape) != (T, D):
+        raise KernelError(f"{who}: expected [{T}, {D}], got {tuple(y.shape)}")
+    return 1, _code(y)
+
+
+def input_conv(n, hist, weights, outs, step):
+    """outs[r][t] = n[t] + causal convolution of n's rows with weights[r] ([D, taps] float32) for one or two readers
+    of the same rows n (float32 [T, D]); rows before the step come from hist (float32 [slots, taps - 1, D]), which
+    is then left holding each sequence's last taps - 1 rows."""
+    _gpu(n, hist, *weights, *outs)
+    T, D = n.shape
+    _f32("n", n)
+    taps = weights[0].shape[1]
+    if not 1 <= len(weights) <= 2 or len(outs) != len(weights) or T != step.n_tokens:
+        raise KernelError("input_conv: one or two readers, an output for each, one row per token of the step")
+    for w, o in zip(weights, outs):
+        _f32("weights", w, D * taps); _contig("out", o)
+        if tuple(o.shape) != (T, D) or o.dtype != outs[0].dtype:
+            raise KernelError("input_conv: outputs are [T, D] of one dtype")
+    if taps > 1:
+        _f32("hist", hist)
+        if tuple(hist.shape[1:]) != (taps - 1, D):
+            raise KernelError(f"input_conv: the history is {tuple(hist.shape)}, expected [slots, {taps - 1}, {D}]")
+    two = len(weights) == 2
+    _call("blm_input_conv", n.data_ptr(), _ptr(hist) if taps > 1 else 0, weights[0].data_ptr(),
+          weights[1].data_ptr() if two else 0, outs[0].data_ptr(), outs[1].data_ptr() if two else 0, len(weights),
+          _code(outs[0]), taps, step.token_seq.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T,
+          step.n_seqs, D, _stream())
+    return outs
+
+
+def residual_add(h, a, b=None, bias=None, copy=None):
+    """h += a (+ b) (+ bias) in float32; copy (if given, [T, D] in any kernel dtype) receives the new h.  a, b: [T, D]
+    or float32 planes [P, T, D]."""
+    _gpu(h, a, b, bias, copy)
+    T, D = h.shape
+    _f32("h", h)
+    pa, ca = _planes("residual_add: a", a, T, D)
+    pb, cb = _planes("residual_add: b", b, T, D) if b is not None else (1, 0)
+    if bias is not None:
+        _f32("bias", bias, D)
+    if copy is not None:
+        _contig("copy", copy)
+        if tuple(copy.shape) != (T, D):
+            raise KernelError("residual_add: the copy is [T, D]")
+    _call("blm_residual_add", h.data_ptr(), a.data_ptr(), ca, pa, _ptr(b), cb, pb, _ptr(bias), _ptr(copy),
+          _code(copy) if copy is not None else 0, T, D, _stream())
+    return h
+
+
+def side_gate(z, table, col0, ids, out, token_source=None):
+    """out[t, j] = gelu_tanh(z[t, j]) * table[token of t, col0 + j]; token_source: None or the step's (rows, cell) of
+    tokens that are still on the device (see embed_gather_from)."""
+    _gpu(z, table, ids, out)
+    T, dim = z.shape
+    _contig("z", z); _contig("table", table); _contig("out", out)
+    _i32("ids", ids, T)
+    if out.shape != z.shape or out.dtype != z.dtype or table.dim() != 2:
+        raise KernelError("side_gate: shapes do not fit")
+    rows = cell = None
+    if token_source is not None:
+        rows, cell = token_source
+        _i32("source_rows", rows, T)
+        if cell.dtype != torch.int64 or cell.numel() != 1:
+            raise KernelError("side_gate: the cell is one int64 on the device")
+    _call("blm_side_gate", z.data_ptr(), _code(z), table.data_ptr(), _code(table), table.shape[1], int(col0), ids.data_ptr(),
+          _ptr(rows), _ptr(cell), table.shape[0], out.data_ptr(), T, dim, _stream())
+    return out
+
+
+def rms_scale(y, w, eps, out):
+    """out = y / sqrt(mean(y^2) + eps) * w as float32 [T, D]; y: [T, D] or float32 planes [P, T, D]."""
+    _gpu(y, w, out)
+    T, D = out.shape
+    _f32("out", out); _f32("w", w, D)
+    planes, code = _planes("rms_scale: y", y, T, D)
+    _call("blm_rms_scale", y.data_ptr(), code, planes, w.data_ptr(), out.data_ptr(), T, D, float(eps), _stream())
+    return out
+
+
+def clamped_glu(gate_up, out, limit, alpha):
+    """g = min(gate, limit), u = clamp(up, -limit, limit): out = g * sigmoid(alpha * g) * (u + 1); gate_up [T, 2 I]."""
+    _gpu(gate_up, out)
+    T, I = out.shape
+    _contig("gate_up", gate_up); _contig("out", out)
+    if tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError("clamped_glu: gate_up is [T, 2 I] in out's dtype")
+    _call("blm_clamped_glu", gate_up.data_ptr(), out.data_ptr(), _code(out), T, I, float(limit), float(alpha), _stream())
+    return out
+
+
+def moe_route(logits, bias, n_experts, top, shared_col, weights):
+    """weights [T, E + 1] float32: for each token the softmax over its `top` largest of (logits[:, :E] + bias) at the
+    chosen experts' places and zero elsewhere; at E the sigmoid of logits[:, shared_col] (shared_col < 0: one)."""
+    _gpu(logits, bias, weights)
+    T = logits.shape[0]
+    _f32("logits", logits); _f32("bias", bias, n_experts); _f32("weights", weights, T * (n_experts + 1))
+    _call("blm_moe_route", logits.data_ptr(), logits.shape[1], bias.data_ptr(), n_experts, top, shared_col,
+          weights.data_ptr(), T, _stream())
+    return weights
+
+
+def moe_gate(gate_up, weights, out, n_experts, expert_inner):
+    """out[t, i] = silu(gate) * up * weights[t, expert of column i] for experts stacked along the columns (expert e at
+    columns e * expert_inner, a shared expert behind them with the weight at E); gate_up [T, 2 I], out [T, I]."""
+    _gpu(gate_up, weights, out)
+    T, I = out.shape
+    _contig("gate_up", gate_up); _contig("out", out)
+    _f32("weights", weights, T * (n_experts + 1))
+    if tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError("moe_gate: gate_up is [T, 2 I] in out's dtype")
+    _call("blm_moe_gate", gate_up.data_ptr(), weights.data_ptr(), out.data_ptr(), _code(out), T, I, n_experts,
+          expert_inner, _stream())
+    return out
+
+
+def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, step, H, dk, dv):
+    """Gated linear attention over proj [T, >= 2 H dk + 2 H dv]: queries, keys, values, output-gate logits;
+    decay_in [T, H dk]: the decays' logits before their bias.  state float32 [slots, H, dk, dv] is read and left
+    updated; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in proj's dtype."""
+    _gpu(proj, decay_in, decay_bias, norm_w, state, o_raw, out)
+    T = proj.shape[0]
+    _f32("o_raw", o_raw, T * H * dv); _f32("decay_bias", decay_bias, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
+    _contig("decay_in", decay_in); _contig("out", out)
+    gates = torch.empty(T, H * dk, dtype=torch.float32, device=proj.device)
+    if proj.stride(1) != 1 or out.dtype != proj.dtype or decay_in.dtype != proj.dtype or tuple(out.shape) != (T, H * dv) \
+            or tuple(decay_in.shape) != (T, H * dk) or tuple(state.shape[1:]) != (H, dk, dv):
+        raise KernelError("gla_scan: shapes do not fit")
+    _call("blm_gla_scan", proj.data_ptr(), _code(proj), proj.stride(0), decay_in.data_ptr(), decay_bias.data_ptr(), float(tau),
+          norm_w.data_ptr(), float(eps), state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(),
+          step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs, H, dk, dv, _stream())
+    return out
+
+
+def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page_size, H, G, dk, dv, write_kv=True):
+    """Bias, rotation of the first `rot` lanes of every query and key head by the token's position (lane i with
+    lane i + rot/2; cos_sin float32 [positions, >= rot/2, 2] rows of exactly rot/2 pairs), queries in place, rotated
+    keys and values into the pages (key pages [pages, G, page, dk], value pages [pages, G, dv, page]).  write_kv
+    False: qkv holds queries only and nothing is stored."""
+    _gpu(qkv, bias, cos_sin, block_table, kcache, vcache)
+    T = qkv.shape[0]
+    if qkv.stride(1) != 1:
+        raise KernelError("qkv_prepare: rows must be contiguous")
+    need = H * dk + (G * (dk + dv) if write_kv else 0)
+    if qkv.shape[1] < need or T != step.n_tokens:
+        raise KernelError(f"qkv_prepare: rows of {qkv.shape[1]}, needs {need}")
+    if bias is not None:
+        _f32("bias", bias, need)
+    if rot:
+        _contig("cos_sin", cos_sin)
+        if cos_sin.dtype != torch.float32 or tuple(cos_sin.shape[1:]) != (rot // 2, 2) or cos_sin.shape[0] <= step.max_position:
+            raise KernelError("qkv_prepare: cos_sin must be float32 [positions, rot/2, 2] and cover the step's positions")
+    if write_kv:
+        _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
+        if kcache.dtype != qkv.dtype or vcache.dtype != qkv.dtype or tuple(kcache.shape[1:]) != (G, page_size, dk) \
+                or tuple(vcache.shape) != (kcache.shape[0], G, dv, page_size):
+            raise KernelError(f"qkv_prepare: pages {tuple(kcache.shape)} / {tuple(vcache.shape)} do not fit")
+    _call("blm_qkv_prepare", qkv.data_ptr(), _code(qkv), qkv.stride(0), _ptr(bias), _ptr(cos_sin) if rot else 0, rot,
+          step.positions.data_ptr(), step.token_seq.data_ptr(), _ptr(block_table) if write_kv else 0,
+          block_table.shape[1] if write_kv else 0, _ptr(kcache) if write_kv else 0, _ptr(vcache) if write_kv else 0,
+          page_size, T, H, G, dk, dv, 1 if write_kv else 0, _stream())
+    return qkv
+
+
+def sink_attn(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, H, G, dk, dv, scale, window):
+    """Attention whose softmax denominator also holds exp(sinks[h]) (sinks None: a plain softmax) and whose weights
+    are mixed between heads by mix [H, H] (None: not mixed) before head h reads the values of its own key-value head.
+    q [T, >= H dk] rows (queries already rotated), out [T, H * dv] in q's dtype."""
+    _gpu(q, out, sinks, mix, block_table, kcache, vcache)
+    T = q.shape[0]
+    _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
+    if q.stride(1) != 1 or out.dtype != q.dtype or kcache.dtype != q.dtype or vcache.dtype != q.dtype:
+        raise KernelError("sink_attn: queries, pages and output share a dtype; rows contiguous")
+    if tuple(out.shape) != (T, H * dv) or tuple(kcache.shape[1:]) != (G, page_size, dk) \
+            or tuple(vcache.shape) != (kcache.shape[0], G, dv, page_size) or T != step.n_tokens:
+        raise KernelError(f"sink_attn: shapes do not fit: out {tuple(out.shape)}, pages {tuple(kcache.shape)} / {tuple(vcache.shape)}")
+    if sinks is not None:
+        _f32("sinks", sinks, H)
+    if mix is not None:
+        _f32("mix", mix, H * H)
+    A = torch.empty(T, H, G if mix is not None else 1, dv, dtype=torch.float32, device=q.device)
+    _call("blm_sink_attn", q.data_ptr(), q.stride(0), out.data_ptr(), _code(q), A.data_ptr(), _ptr(sinks), _ptr(mix),
+          step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+          kcache.data_ptr(), vcache.data_ptr(), page_size, T, H, G, dk, dv, float(scale), int(window), _stream())
     return out

@@ -1,0 +1,355 @@
+// Kernels around the sublayers of a layer whose mixer and feed-forward read the same normalised rows side by
+// side: a short causal convolution added to what each sublayer reads, the float residual add of both results,
+// a gated per-token side input, an RMS norm that hands on a float delta, a clamped gated activation, and the
+// routing and gating of a mixture of experts whose experts run as one stacked product.
+#include "common.h"
+
+#define PB_MAX_TAPS 16
+#define PB_MAX_READERS 4
+#define PB_MAX_TOP 16
+
+__device__ __forceinline__ float pb_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------
+// out_r[t][c] = n[t][c] + sum_k w_r[c][k] * n(t - taps + 1 + k)[c] for every reader r; rows before the step come
+// from hist [slots][taps-1][D] (oldest first; zeros in a fresh slot stand for "before the sequence").  n is the
+// float output of the norm; padding tokens (sequence -1) give zeros.
+// ---------------------------------------------------------------------------------------
+struct PbReaders {
+  const float* w[PB_MAX_READERS];   // [D][taps]
+  void* out[PB_MAX_READERS];        // [T][D]
+};
+
+template <typename TO>
+__global__ void input_conv_kernel(const float* __restrict__ n, const float* __restrict__ hist, PbReaders rd, int readers,
+                                  int taps, const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
+                                  const int* __restrict__ seq_slots, int D) {
+  const int t = blockIdx.x;
+  const int b = token_seq[t];
+  if (b < 0) {
+    for (int c = threadIdx.x; c < D; c += blockDim.x)
+      for (int r = 0; r < readers; ++r) ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(0.f);
+    return;
+  }
+  const int start = cu_seqlens[b], slot = seq_slots[b];
+  const int off = t - start;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) {
+    float x[PB_MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < PB_MAX_TAPS; ++k) {
+      if (k < taps) {
+        const int src = off - (taps - 1) + k;
+        x[k] = src >= 0 ? n[(size_t)(start + src) * D + c]
+                        : (slot >= 0 ? hist[((size_t)slot * (taps - 1) + (taps - 1 + src)) * D + c] : 0.f);
+      }
+    }
+    for (int r = 0; r < readers; ++r) {
+      const float* w = rd.w[r] + (size_t)c * taps;
+      float a = 0.f;
+#pragma unroll
+      for (int k = 0; k < PB_MAX_TAPS; ++k)
+        if (k < taps) a = fmaf(w[k], x[k], a);
+      ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(n[(size_t)t * D + c] + a);
+    }
+  }
+}
+
+// the history after the step: each sequence's last taps-1 rows, from the step's rows and, where the step brought
+// fewer, from the old history; a thread reads all it needs before it writes.  Runs after the convolution.
+__global__ void input_history_kernel(const float* __restrict__ n, int taps, float* __restrict__ hist,
+                                     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int D) {
+  const int b = blockIdx.x;
+  const int slot = seq_slots[b];
+  const int start = cu_seqlens[b], cnt = cu_seqlens[b + 1] - start;
+  if (slot < 0 || cnt <= 0) return;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < D; c += gridDim.y * blockDim.x) {
+    float keep[PB_MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < PB_MAX_TAPS; ++k) {
+      if (k < taps - 1) {
+        const int src = cnt - (taps - 1) + k;
+        keep[k] = src >= 0 ? n[(size_t)(start + src) * D + c] : hist[((size_t)slot * (taps - 1) + (k + cnt)) * D + c];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < PB_MAX_TAPS; ++k)
+      if (k < taps - 1) hist[((size_t)slot * (taps - 1) + k) * D + c] = keep[k];
+  }
+}
+
+extern "C" int blm_input_conv(const float* n, float* hist, const float* w0, const float* w1, void* out0, void* out1,
+                              int readers, int out_dtype, int taps, const int* token_seq, const int* cu_seqlens, const int* seq_slots,
+                              int T, int B, int D, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && B > 0 && D > 0, "input_conv: bad sizes T=%d B=%d D=%d", T, B, D);
+  BLM_REQUIRE(taps >= 1 && taps <= PB_MAX_TAPS, "input_conv: %d taps (1 to %d)", taps, PB_MAX_TAPS);
+  BLM_REQUIRE(readers >= 1 && readers <= 2, "input_conv: %d readers (1 or 2)", readers);
+  const float* weights[2] = {w0, w1};
+  void* outs[2] = {out0, out1};
+  BLM_REQUIRE(taps == 1 || hist, "input_conv: the history is missing");
+  PbReaders rd;
+  for (int r = 0; r < readers; ++r) {
+    BLM_REQUIRE(weights[r] && outs[r], "input_conv: reader %d lacks its weights or output", r);
+    rd.w[r] = weights[r];
+    rd.out[r] = outs[r];
+  }
+  const int threads = D >= 1024 ? 512 : (D >= 256 ? 256 : 128);
+  if (out_dtype == BLM_F32)
+    hipLaunchKernelGGL(input_conv_kernel<float>, dim3(T), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+                       cu_seqlens, seq_slots, D);
+  else if (out_dtype == BLM_BF16)
+    hipLaunchKernelGGL(input_conv_kernel<bf16>, dim3(T), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+                       cu_seqlens, seq_slots, D);
+  else
+    return blm_fail("input_conv: unsupported dtype %d", out_dtype);
+  BLM_LAUNCH_CHECK("input_conv");
+  if (taps > 1) {
+    hipLaunchKernelGGL(input_history_kernel, dim3(B, (D + 255) / 256), dim3(256), 0, stream, n, taps, hist, cu_seqlens,
+                       seq_slots, D);
+    BLM_LAUNCH_CHECK("input_history");
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// h[t] += a[t] + b[t] (+ bias), in float; copy[t] = the new h[t] in the activation dtype.  a and b: [T][D] in
+// the activation dtype or float planes [P][T][D] that are summed in order; b may be missing.
+// ---------------------------------------------------------------------------------------
+template <typename TA, typename TB, typename TO>
+__global__ void residual_add_kernel(float* __restrict__ h, const TA* __restrict__ a, int a_planes, const TB* __restrict__ b,
+                                    int b_planes, const float* __restrict__ bias, TO* __restrict__ copy, long long n, int D) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    float da = 0.f, db = 0.f;
+    for (int p = 0; p < a_planes; ++p) da += to_float(a[(size_t)p * n + e]);
+    if (bias) da += bias[e % D];
+    if (b)
+      for (int p = 0; p < b_planes; ++p) db += to_float(b[(size_t)p * n + e]);
+    const float v = h[e] + (da + db);
+    h[e] = v;
+    if (copy) copy[e] = from_float<TO>(v);
+  }
+}
+
+extern "C" int blm_residual_add(float* h, const void* a, int a_dtype, int a_planes, const void* b, int b_dtype, int b_planes,
+                                const float* bias, void* copy, int copy_dtype, int T, int D, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0 && a && a_planes >= 1 && b_planes >= 1, "residual_add: bad sizes T=%d D=%d", T, D);
+  const long long n = (long long)T * D;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (!b) b_dtype = a_dtype;
+  if (!copy) copy_dtype = BLM_F32;
+#define PB_RA(TA, TB, TO)                                                                                            \
+  hipLaunchKernelGGL((residual_add_kernel<TA, TB, TO>), dim3(blocks), dim3(256), 0, stream, h, (const TA*)a, a_planes, \
+                     (const TB*)b, b_planes, bias, (TO*)copy, n, D)
+#define PB_RA_O(TA, TB)                       \
+  do {                                        \
+    if (copy_dtype == BLM_F32) PB_RA(TA, TB, float); \
+    else PB_RA(TA, TB, bf16);                 \
+  } while (0)
+  BLM_REQUIRE((a_dtype == BLM_F32 || a_dtype == BLM_BF16) && (b_dtype == BLM_F32 || b_dtype == BLM_BF16) &&
+                  (copy_dtype == BLM_F32 || copy_dtype == BLM_BF16), "residual_add: unsupported dtypes");
+  if (a_dtype == BLM_F32 && b_dtype == BLM_F32) PB_RA_O(float, float);
+  else if (a_dtype == BLM_F32) PB_RA_O(float, bf16);
+  else if (b_dtype == BLM_F32) PB_RA_O(bf16, float);
+  else PB_RA_O(bf16, bf16);
+#undef PB_RA_O
+#undef PB_RA
+  BLM_LAUNCH_CHECK("residual_add");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Side input per token: out[t][j] = gelu_tanh(z[t][j]) * table[token of t][col0 + j].  The token of row t is
+// ids[t], or (as for the embedding) element source_rows[t] of the array whose address is in the source cell.
+// ---------------------------------------------------------------------------------------
+template <typename TA, typename TW>
+__global__ void side_gate_kernel(const TA* __restrict__ z, const TW* __restrict__ table, int table_ld, int col0,
+                                 const int* __restrict__ ids, const int* __restrict__ source_rows,
+                                 const int* const* __restrict__ source, int V, TA* __restrict__ out, int T, int dim) {
+  const long long n = (long long)T * dim;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const int t = (int)(e / dim), j = (int)(e - (long long)t * dim);
+    int id = ids[t];
+    if (source_rows) {
+      const int r = source_rows[t];
+      if (r >= 0) id = (*source)[r];
+    }
+    float v;
+    if ((unsigned)id >= (unsigned)V) {
+      v = __builtin_nanf("");
+    } else {
+      const float x = to_float(z[e]);
+      const float g = 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+      v = g * to_float(table[(size_t)id * table_ld + col0 + j]);
+    }
+    out[e] = from_float<TA>(v);
+  }
+}
+
+extern "C" int blm_side_gate(const void* z, int dtype, const void* table, int table_dtype, int table_ld, int col0,
+                             const int* ids, const int* source_rows, const void* source_cell, int V, void* out, int T,
+                             int dim, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && dim > 0 && V > 0 && col0 >= 0 && col0 + dim <= table_ld, "side_gate: bad sizes T=%d dim=%d", T, dim);
+  BLM_REQUIRE((source_rows == nullptr) == (source_cell == nullptr), "side_gate: rows and cell of a token source come together");
+  const long long n = (long long)T * dim;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  const int* const* cell = (const int* const*)source_cell;
+#define PB_SG(TA, TW)                                                                                                 \
+  hipLaunchKernelGGL((side_gate_kernel<TA, TW>), dim3(blocks), dim3(256), 0, stream, (const TA*)z, (const TW*)table, \
+                     table_ld, col0, ids, source_rows, cell, V, (TA*)out, T, dim)
+  if (dtype == BLM_F32 && table_dtype == BLM_F32) PB_SG(float, float);
+  else if (dtype == BLM_BF16 && table_dtype == BLM_BF16) PB_SG(bf16, bf16);
+  else if (dtype == BLM_F32 && table_dtype == BLM_BF16) PB_SG(float, bf16);
+  else return blm_fail("side_gate: unsupported dtypes %d / %d", dtype, table_dtype);
+#undef PB_SG
+  BLM_LAUNCH_CHECK("side_gate");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// out[t] = y[t] / sqrt(mean(y[t]^2) + eps) * w, float out; y in the activation dtype or float planes that are summed.
+// ---------------------------------------------------------------------------------------
+template <typename TY>
+__global__ void rms_scale_kernel(const TY* __restrict__ y, int planes, size_t plane_stride, const float* __restrict__ w,
+                                 float* __restrict__ out, int D, float eps) {
+  extern __shared__ float row[];
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float v = 0.f;
+    for (int p = 0; p < planes; ++p) v += to_float(y[p * plane_stride + (size_t)t * D + d]);
+    row[d] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum<true>(ss, red) / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) out[(size_t)t * D + d] = row[d] * inv * w[d];
+}
+
+extern "C" int blm_rms_scale(const void* y, int dtype, int planes, const float* w, float* out, int T, int D, float eps,
+                             hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && D > 0 && D <= 16384 && planes >= 1, "rms_scale: bad sizes T=%d D=%d", T, D);
+  const int threads = D >= 1024 ? 512 : (D >= 256 ? 256 : 128);
+  const size_t stride = (size_t)T * D;
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(rms_scale_kernel<float>, dim3(T), dim3(threads), (size_t)D * sizeof(float), stream, (const float*)y,
+                       planes, stride, w, out, D, eps);
+  else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(rms_scale_kernel<bf16>, dim3(T), dim3(threads), (size_t)D * sizeof(float), stream, (const bf16*)y,
+                       planes, stride, w, out, D, eps);
+  else
+    return blm_fail("rms_scale: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("rms_scale");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Clamped gated activation: g = min(gate, limit), u = clamp(up, -limit, limit); out = g * sigmoid(alpha g) * (u + 1).
+// gate_up [T][2 I]: gate columns, then up columns.
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void clamped_glu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ out, long long n, int I, float limit,
+                                   float alpha) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / I;
+    const int i = (int)(e - t * I);
+    const float g = fminf(to_float(gate_up[(size_t)t * 2 * I + i]), limit);
+    const float u = fminf(fmaxf(to_float(gate_up[(size_t)t * 2 * I + I + i]), -limit), limit);
+    out[e] = from_float<TA>(g * pb_sigmoid(alpha * g) * (u + 1.0f));
+  }
+}
+
+extern "C" int blm_clamped_glu(const void* gate_up, void* out, int dtype, int T, int I, float limit, float alpha,
+                               hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && I > 0 && limit > 0.f, "clamped_glu: bad sizes T=%d I=%d limit=%g", T, I, (double)limit);
+  const long long n = (long long)T * I;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, (float*)out, n, I, limit, alpha);
+  else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, n, I, limit, alpha);
+  else
+    return blm_fail("clamped_glu: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("clamped_glu");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Routing of a mixture of experts.  logits [T][ld] float: E router logits, then (if shared) one logit of the
+// shared expert's gate; bias [E] is added.  The `top` largest logits are chosen (the lower index wins a tie);
+// their weights are the softmax over the chosen logits only.  weights [T][E + 1] float: an expert's weight or 0,
+// and at E the shared expert's sigmoid gate (1 if there is no gate logit).
+// ---------------------------------------------------------------------------------------
+__global__ void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias, int E, int top,
+                                 int shared_col, float* __restrict__ weights, int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (size_t)t * ld;
+  float* w = weights + (size_t)t * (E + 1);
+  int chosen[PB_MAX_TOP];
+  float val[PB_MAX_TOP];
+  for (int e = 0; e < E; ++e) w[e] = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+      const float v = z[e] + bias[e];
+      if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
+    }
+    chosen[k] = best;
+    val[k] = bv;
+  }
+  float sum = 0.f;
+  const float largest = val[0];
+  for (int k = 0; k < top; ++k) { val[k] = expf(val[k] - largest); sum += val[k]; }
+  for (int k = 0; k < top; ++k) w[chosen[k]] = val[k] / sum;
+  w[E] = shared_col >= 0 ? pb_sigmoid(z[shared_col]) : 1.0f;
+}
+
+extern "C" int blm_moe_route(const float* logits, int ld, const float* bias, int E, int top, int shared_col, float* weights,
+                             int T, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && E > 0 && top >= 1 && top <= E && top <= PB_MAX_TOP && ld >= E && shared_col < ld,
+              "moe_route: bad sizes T=%d experts=%d top=%d (top at most %d)", T, E, top, PB_MAX_TOP);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 127) / 128), dim3(128), 0, stream, logits, ld, bias, E, top, shared_col, weights, T);
+  BLM_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// The experts' gated activations, each scaled by its expert's weight for the token, for experts that run as one
+// stacked product.  gate_up [T][2 I] with I = E * ffe + ffs columns of gates (expert e at e * ffe, the shared expert
+// behind them), then as many of ups.  out[t][i] = silu(gate) * up * weights[t][expert of column i].
+template <typename TA>
+__global__ void moe_gate_kernel(const TA* __restrict__ gate_up, const float* __restrict__ weights, TA* __restrict__ out,
+                                long long n, int I, int E, int ffe) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / I;
+    const int i = (int)(e - t * I);
+    const int ex = i / ffe < E ? i / ffe : E;
+    const float w = weights[(size_t)t * (E + 1) + ex];
+    float v = 0.f;
+    if (w != 0.f) {
+      const float g = to_float(gate_up[(size_t)t * 2 * I + i]), u = to_float(gate_up[(size_t)t * 2 * I + I + i]);
+      v = g * pb_sigmoid(g) * u * w;
+    }
+    out[e] = from_float<TA>(v);
+  }
+}
+
+extern "C" int blm_moe_gate(const void* gate_up, const float* weights, void* out, int dtype, int T, int I, int E, int ffe,
+                            hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && E > 0 && ffe > 0 && I >= E * ffe, "moe_gate: bad sizes T=%d I=%d experts=%d of %d", T, I, E, ffe);
+  const long long n = (long long)T * I;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(moe_gate_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, weights, (float*)out, n, I, E, ffe);
+  else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(moe_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)gate_up, weights, (bf16*)out, n, I, E, ffe);
+  else
+    return blm_fail("moe_gate: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("moe_gate");
+  return 0;
+}

@@ -170,35 +170,40 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   }
 }
 
-// out[t][h][j] = o_raw[t][h][j] / sqrt(mean_j(o_raw^2) + eps) * norm_w[j] (* sigmoid(gate[t][h][j])); one wavefront
-// per (token, head).  Rows of padding tokens hold whatever o_raw holds (the caller clears it).
+// out[t][h][j] = o_raw[t][h][j] / sqrt(mean_j(o_raw^2) + eps) * norm_w[j] (* f(gate[t][h * dv + j])); one wavefront
+// per (token, head).  gate rows are gate_ld elements apart; f is the sigmoid (gate_mode 1) or SiLU (gate_mode 2).
+// Rows of padding tokens hold whatever o_raw holds (the caller clears it).
 template <typename TA>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     head_norm_kernel(const float* __restrict__ o_raw, const float* __restrict__ norm_w, const TA* __restrict__ gate,
-                     TA* __restrict__ out, long long n_items, int dv, float eps) {
+                     int gate_ld, int gate_mode, int H, TA* __restrict__ out, long long n_items, int dv, float eps) {
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long item = (long long)blockIdx.x * SCAN_WAVES + wave;
   if (item >= n_items) return;
   const float* src = o_raw + (size_t)item * dv;
+  const TA* grow = gate ? gate + (size_t)(item / H) * gate_ld + (size_t)(item % H) * dv : nullptr;
   float ss = 0.f;
   for (int j = lane; j < dv; j += BLM_WAVE) ss = fmaf(src[j], src[j], ss);
   const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
   for (int j = lane; j < dv; j += BLM_WAVE) {
     float v = src[j] * inv * norm_w[j];
-    if (gate) v *= blm_sigmoid(to_float(gate[(size_t)item * dv + j]));
+    if (grow) {
+      const float z = to_float(grow[j]);
+      v *= gate_mode == 2 ? blm_silu(z) : blm_sigmoid(z);
+    }
     out[(size_t)item * dv + j] = from_float<TA>(v);
   }
 }
 
-static int launch_head_norm(const float* o_raw, const float* norm_w, const void* gate, void* out, int dtype, long long items,
-                            int dv, float eps, hipStream_t stream) {
+static int launch_head_norm(const float* o_raw, const float* norm_w, const void* gate, int gate_ld, int gate_mode, int H,
+                            void* out, int dtype, long long items, int dv, float eps, hipStream_t stream) {
   const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(head_norm_kernel<float>, dim3(blocks), dim3(SCAN_WAVES * BLM_WAVE), 0, stream, o_raw, norm_w,
-                       (const float*)gate, (float*)out, items, dv, eps);
+                       (const float*)gate, gate_ld, gate_mode, H, (float*)out, items, dv, eps);
   else
     hipLaunchKernelGGL(head_norm_kernel<bf16>, dim3(blocks), dim3(SCAN_WAVES * BLM_WAVE), 0, stream, o_raw, norm_w,
-                       (const bf16*)gate, (bf16*)out, items, dv, eps);
+                       (const bf16*)gate, gate_ld, gate_mode, H, (bf16*)out, items, dv, eps);
   BLM_LAUNCH_CHECK("head_norm");
   return 0;
 }
@@ -269,7 +274,7 @@ extern "C" int blm_hgrn2_scan(const void* proj, int dtype, int ld, const float* 
   BLM_SCAN_PICK(BLM_HG);
 #undef BLM_HG
   BLM_LAUNCH_CHECK("hgrn2_scan");
-  return launch_head_norm(o_raw, norm_w, nullptr, out, dtype, (long long)T * H, dv, eps, stream);
+  return launch_head_norm(o_raw, norm_w, nullptr, 0, 0, H, out, dtype, (long long)T * H, dv, eps, stream);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -550,5 +555,159 @@ extern "C" int blm_delta_scan(const float* qkv, int C, const void* beta_src, int
   BLM_SCAN_PICK(BLM_DS);
 #undef BLM_DS
   BLM_LAUNCH_CHECK("delta_scan");
-  return launch_head_norm(o_raw, norm_w, gate_in, out, dtype, (long long)T * H, dv, eps, stream);
+  return launch_head_norm(o_raw, norm_w, gate_in, H * dv, 1, H, out, dtype, (long long)T * H, dv, eps, stream);
+}
+
+// ---------------------------------------------------------------------------------------
+// Gated linear attention.  proj [T][ld]: q at column 0 (H*dk), k at H*dk (H*dk), v at 2*H*dk (H*dv), the output
+// gate's logits at 2*H*dk + H*dv (H*dv).  decay_in [T][H*dk]: the decay's logits before their bias.
+//   alpha = sigmoid(decay_in + bias)^(1/tau) = exp(-softplus(-(decay_in + bias)) / tau)
+//   S = diag(alpha) S + k v^T;  o = S^T (q * dk^-1/2)
+// then out = o / sqrt(mean(o^2) + eps) * norm_w * silu(gate) by head_norm_kernel.
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void gla_gates_kernel(const TA* __restrict__ decay_in, const float* __restrict__ bias, float inv_tau,
+                                 float* __restrict__ gates, long long n, int HK) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride)
+    gates[e] = expf(-blm_softplus(-(to_float(decay_in[e]) + bias[e % HK])) * inv_tau);
+}
+
+template <typename TA, int ROWS, int LPC>
+__global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
+    gla_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates, float q_scale,
+                    float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
+                    const int* __restrict__ seq_slots, int H, int dk, int dv, int col_groups, long long n_items) {
+  extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][decay | k | q][vec], [chunk][16 values]
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const long long item = (long long)blockIdx.x * (blockDim.x / BLM_WAVE) + wave;
+  if (item >= n_items) return;
+  const int cg = (int)(item % col_groups);
+  const int h = (int)((item / col_groups) % H);
+  const int b = (int)(item / ((long long)col_groups * H));
+  const int slot = seq_slots[b];
+  const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+  if (slot < 0 || t1 <= t0) return;
+  constexpr int COLS = BLM_WAVE / LPC;
+  const int g = LPC == 4 ? lane >> 4 : lane & 15, cl = LPC == 4 ? lane & 15 : lane >> 4;
+  const int col = cg * COLS + cl;
+  const bool own = col < dv;
+  constexpr int dkp = ROWS * LPC;
+  constexpr int vec = LPC * (ROWS + 4);
+  float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (3 * vec + 2 * SCAN_COLS);
+  float* v_sm = base + SCAN_CHUNK * 3 * vec;
+  float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
+  float S[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) {
+    const int i = g * ROWS + r;
+    S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
+  }
+  constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
+  float raw_d[SCAN_CHUNK][PER], raw_k[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK];
+  auto fetch = [&](int tc) {
+#pragma unroll
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tc + tt < t1) {
+        const int t = tc + tt;
+        const TA* row = proj + (size_t)t * ld;
+        const float* gr = gates + (size_t)t * H * dk;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dk) {
+            raw_d[tt][k] = gr[h * dk + i];
+            raw_k[tt][k] = to_float(row[(size_t)H * dk + h * dk + i]);
+            raw_q[tt][k] = to_float(row[h * dk + i]) * q_scale;
+          }
+        }
+        v_in[tt] = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
+      }
+    }
+  };
+  fetch(t0);
+  for (int tc = t0; tc < t1; tc += SCAN_CHUNK) {
+    const int n = min(SCAN_CHUNK, t1 - tc);
+#pragma unroll
+    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+      if (tt < n) {
+        if (g == 0) v_sm[tt * 2 * SCAN_COLS + cl] = v_in[tt];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+          const int i = lane + k * BLM_WAVE;
+          if (i < dkp) {
+            const int at = scan_place<ROWS>(i);
+            base[(tt * 3) * vec + at] = i < dk ? raw_d[tt][k] : 0.f;
+            base[(tt * 3 + 1) * vec + at] = i < dk ? raw_k[tt][k] : 0.f;
+            base[(tt * 3 + 2) * vec + at] = i < dk ? raw_q[tt][k] : 0.f;
+          }
+        }
+      }
+    }
+    if (tc + SCAN_CHUNK < t1) fetch(tc + SCAN_CHUNK);     // the next chunk's inputs travel while this one runs
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll 1
+    for (int tt = 0; tt < n; ++tt) {
+      const float* bg = base + (tt * 3) * vec + g * (ROWS + 4);
+      const float vv = v_sm[tt * 2 * SCAN_COLS + cl];
+      float o = 0.f;
+#pragma unroll
+      for (int r = 0; r < ROWS; r += 4) {
+        const float4 d4 = *reinterpret_cast<const float4*>(bg + r);
+        const float4 k4 = *reinterpret_cast<const float4*>(bg + vec + r);
+        const float4 q4 = *reinterpret_cast<const float4*>(bg + 2 * vec + r);
+        const float d[4] = {d4.x, d4.y, d4.z, d4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, q[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          S[r + e] = fmaf(d[e], S[r + e], kk[e] * vv);
+          o = fmaf(S[r + e], q[e], o);
+        }
+      }
+      o = column_sum<LPC>(o);
+      if (own && g == 0) o_raw[(size_t)(tc + tt) * H * dv + h * dv + col] = o;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (own) {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = g * ROWS + r;
+      if (i < dk) S_g[(size_t)i * dv + col] = S[r];
+    }
+  }
+}
+
+extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* decay_in, const float* decay_bias, float tau,
+                            const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
+                            const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv,
+                            hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && B > 0 && H > 0 && tau > 0.f, "gla_scan: bad sizes T=%d B=%d H=%d tau=%g", T, B, H, (double)tau);
+  BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "gla_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
+  BLM_REQUIRE(ld >= 2 * H * dk + 2 * H * dv, "gla_scan: rows of %d are too short", ld);
+  BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "gla_scan: unsupported dtype %d", dtype);
+  {
+    const long long n = (long long)T * H * dk;
+    const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    if (dtype == BLM_F32)
+      hipLaunchKernelGGL(gla_gates_kernel<float>, dim3(gblocks), dim3(256), 0, stream, (const float*)decay_in, decay_bias, 1.0f / tau, gates, n, H * dk);
+    else
+      hipLaunchKernelGGL(gla_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)decay_in, decay_bias, 1.0f / tau, gates, n, H * dk);
+    BLM_LAUNCH_CHECK("gla_gates");
+  }
+  const float q_scale = 1.0f / sqrtf((float)dk);
+#define BLM_GLA(ROWS, LPC)                                                                                                \
+  const int col_groups = (dv + 64 / LPC - 1) / (64 / LPC);                                                                \
+  const long long items = (long long)B * H * col_groups;                                                                  \
+  const ScanLaunch sl = scan_launch(ROWS, LPC, 3, items);                                                                 \
+  if (dtype == BLM_F32)                                                                                                   \
+    hipLaunchKernelGGL((gla_scan_kernel<float, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
+                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                       \
+  else                                                                                                                    \
+    hipLaunchKernelGGL((gla_scan_kernel<bf16, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
+                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
+  BLM_SCAN_PICK(BLM_GLA);
+#undef BLM_GLA
+  BLM_LAUNCH_CHECK("gla_scan");
+  const char* gate = (const char*)proj + (size_t)(2 * H * dk + H * dv) * (dtype == BLM_F32 ? 4 : 2);
+  return launch_head_norm(o_raw, norm_w, gate, ld, 2, H, out, dtype, (long long)T * H, dv, eps, stream);
 }

@@ -5,13 +5,18 @@ from .base import (Block, FeedForward, KVNeed, Mixer, Norm, Part, PartSpec, Posi
                    TensorSpec)
 from .block import PreNormBlock
 from .channel_delta import ChannelDelta
+from .clamped_glu import ClampedGLU
 from .dense_xielu import DenseXielu
 from .embedding import Embedding, LMHead
+from .gla import GatedLinearAttention
 from .hgrn2 import HGRN2
 from .latent_attention import LatentAttention
 from .norm_layer import LayerNorm
 from .norm_rms import RMSNorm
+from .parallel import CausalConvInput, ParallelBlock, ParallelMixerBlock, TokenSide
 from .rope import RotaryEncoding
+from .routed_experts import RoutedExperts
+from .sink_attention import SinkAttention
 from .streams import HyperBlock, HyperConnection, HyperMixerBlock
 from .swiglu import SwiGLU
 
@@ -30,3 +35,11 @@ registry.register_part("norm", "layernorm", LayerNorm)
 registry.register_part("connection", "hyper", HyperConnection)
 registry.register_part("block", "hyper", HyperBlock)
 registry.register_part("block", "hyper_mixer_only", HyperMixerBlock)
+registry.register_part("mixer", "gla", GatedLinearAttention)
+registry.register_part("mixer", "sink_attention", SinkAttention)
+registry.register_part("feed_forward", "clamped_glu", ClampedGLU)
+registry.register_part("feed_forward", "routed_experts", RoutedExperts)
+registry.register_part("connection", "causal_conv", CausalConvInput)
+registry.register_part("connection", "token_side", TokenSide)
+registry.register_part("block", "parallel", ParallelBlock)
+registry.register_part("block", "parallel_mixer_only", ParallelMixerBlock)

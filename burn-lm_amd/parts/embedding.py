@@ -13,7 +13,7 @@ from .base import Part, TensorSpec
 
 class Embedding(Part):
     """params: vocab, width, copies (default 1; more: the residual starts as that many equal streams,
-    [tokens, copies, width]).  names: weight."""
+    [tokens, copies, width]), scale (default 1: every row is multiplied by it).  names: weight."""
     graph_safe = True
 
     def tensor_specs(self):
@@ -22,6 +22,7 @@ class Embedding(Part):
     def bind(self, tensors, rt):
         self.rt = rt
         self.table = tensors[self.names["weight"]].contiguous()
+        self.scale = float(self.params.get("scale", 1.0))
 
     def step_bytes(self, rows):
         return rows * self.params["width"] * self.table.element_size()      # the rows that are looked up
@@ -33,14 +34,14 @@ class Embedding(Part):
 
     def forward(self, ids):
         h = self._rows(ids)
-        return self.rt.ops.embed_gather(self.table, ids, h)
+        return self.rt.ops.embed_gather(self.table, ids, h, self.scale)
 
     def forward_from(self, ids, source_rows, source_cell):
         """The same where some tokens are still on the device: row t is element source_rows[t] of the
         array whose address is in source_cell, where source_rows[t] >= 0.  An embedding without this
         method gets its tokens gathered by a separate launch before the step."""
         h = self._rows(ids)
-        return self.rt.ops.embed_gather_from(self.table, ids, source_rows, source_cell, h)
+        return self.rt.ops.embed_gather_from(self.table, ids, source_rows, source_cell, h, self.scale)
 
 
 class LMHead(Part):

@@ -42,6 +42,7 @@ class LayerNorm(Norm):
         self.eps = float(self.params["eps"])
         self.streams = int(self.params.get("streams", 1))
         self.out_scale = float(self.params.get("out_scale", 1.0))
+        self._ones = None     # the trivial layer scale, mixing matrix and write coefficient of a plain delta
 
     def step_bytes(self, rows):
         return 2 * self.gamma.numel() * 4
@@ -58,12 +59,14 @@ class LayerNorm(Norm):
                                         pending=None if pending is None else pending.as_tuple(), rows=rows,
                                         write_x=write_h, out_scale=self.out_scale, stash=stash)
 
-    def add_norm(self, h, delta, rows=None, write_h=True):
-        """The norm of the sum of the streams, after `delta` (None, or a Pending) has been written into them."""
+    def add_norm(self, h, delta, rows=None, write_h=True, out_dtype=None):
+        """The norm of the sum of the streams, after `delta` (None, a Pending, or with one stream a plain result:
+        [tokens, width] or float32 planes) has been written into them; out_dtype: the activation dtype unless given."""
         if delta is not None and not isinstance(delta, Pending):
             if self.streams != 1:
                 raise ValueError("a plain delta can only be added to a residual of one stream")
-            d = h.shape[-1]
-            one = torch.ones(1, dtype=torch.float32, device=h.device)
-            delta = Pending(delta, torch.ones(d, dtype=torch.float32, device=h.device), one.view(1, 1), one)
-        return self.read_streams(h, delta, None, self.rt.dtype, rows=rows, write_h=write_h)
+            if self._ones is None or self._ones[0].device != h.device:
+                one = torch.ones(1, dtype=torch.float32, device=h.device)
+                self._ones = (torch.ones(h.shape[-1], dtype=torch.float32, device=h.device), one.view(1, 1), one)
+            delta = Pending(delta, *self._ones)
+        return self.read_streams(h, delta, None, out_dtype or self.rt.dtype, rows=rows, write_h=write_h)

@@ -1,0 +1,120 @@
+"""Grouped-query attention with projection biases, a sliding window, a softmax sink and head mixing.
+
+``q, k, v = W x + b``; the first ``rot_dims`` lanes of every query and key head are turned by the token's position
+(lane i with lane i + rot_dims/2, angle ``p * base^(-2i/rot_dims)``), the rest pass; rotated keys and the values
+go into the paged cache.  ``score = q . k * scale``; query i sees key j while ``0 <= i - j < window`` (window 0:
+every earlier key).  The softmax's denominator also holds ``exp(sink_h)``, a learned logit per head without key
+or value.  The heads' weights are then mixed, ``w'_h = sum_g talk[h, g] w_g``, and head h applies its mixed
+weights to the values of its own key-value head.  Keys and values may differ in head size.  A layer that
+borrows (``borrows=True``) has no key and value projections and reads the keys (as cached, rotated) and values
+that an earlier layer keeps, with queries, window, sink and mixing of its own.  Scores, softmax and the mixing
+are float32 in every mode."""
+from __future__ import annotations
+
+import torch
+
+from .base import KVNeed, Mixer, TensorSpec
+
+
+class SinkAttention(Mixer):
+    """params: width, heads, kv_heads, dim, vdim, scale, window (0: all keys), cache_window (what the cache keeps:
+    the largest window of this layer and of the layers that borrow from it; default window), rot_dims, position
+    (a rotary encoding whose table has rot_dims/2 pairs; given by the model builder), borrows, sink, talk (whether
+    the layer has them; default True).
+    names: q, q_bias, o, o_bias, sink, talk and, unless the layer borrows, k, k_bias, v, v_bias."""
+    graph_safe = True
+
+    def _flags(self):
+        p = self.params
+        return bool(p.get("borrows")), p.get("sink", True), p.get("talk", True)
+
+    def tensor_specs(self):
+        p, n = self.params, self.names
+        d, H, G, dk, dv = p["width"], p["heads"], p["kv_heads"], p["dim"], p["vdim"]
+        borrows, sink, talk = self._flags()
+        specs = {n["q"]: TensorSpec((H * dk, d)), n["q_bias"]: TensorSpec((H * dk,)),
+                 n["o"]: TensorSpec((d, H * dv)), n["o_bias"]: TensorSpec((d,))}
+        if sink:
+            specs[n["sink"]] = TensorSpec((H,))
+        if talk:
+            specs[n["talk"]] = TensorSpec((H, H))
+        if not borrows:
+            specs.update({n["k"]: TensorSpec((G * dk, d)), n["k_bias"]: TensorSpec((G * dk,)),
+                          n["v"]: TensorSpec((G * dv, d)), n["v_bias"]: TensorSpec((G * dv,))})
+        return specs
+
+    def cache_need(self):
+        p = self.params
+        return KVNeed(p["kv_heads"], p["dim"], int(p.get("cache_window", p.get("window", 0))), value_dim=p["vdim"])
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        p, n = self.params, self.names
+        self.H, self.G, self.dk, self.dv = p["heads"], p["kv_heads"], p["dim"], p["vdim"]
+        if self.H % self.G:
+            raise ValueError(f"{self.H} heads are no multiple of {self.G} key-value heads")
+        self.scale, self.window, self.rot = float(p["scale"]), int(p.get("window", 0)), int(p.get("rot_dims", 0))
+        self.borrows, sink, talk = self._flags()
+        self.position = p.get("position")
+        if self.rot and (self.position is None or self.rot % 2 or self.rot > self.dk):
+            raise ValueError("rot_dims must be even, at most the key head size, and come with a rotary encoding")
+        roles = ("q",) if self.borrows else ("q", "k", "v")
+        ws = [tensors[n[r]] for r in roles]
+        if len({w.dtype for w in ws}) != 1:
+            ws = [w.float() for w in ws]
+        rows = sum(w.shape[0] for w in ws)
+        if rows % 8:
+            ws.append(torch.zeros(8 - rows % 8, ws[0].shape[1], dtype=ws[0].dtype, device=ws[0].device))
+        self.w_in = rt.weight(torch.cat(ws, dim=0))
+        self.bias_in = torch.cat([tensors[n[r + "_bias"]].float() for r in roles]).contiguous()
+        self.w_o = rt.weight(tensors[n["o"]])
+        self.output_bias = tensors[n["o_bias"]].float().contiguous()
+        self.sinks = tensors[n["sink"]].float().contiguous() if sink else None
+        self.talk = tensors[n["talk"]].float().contiguous() if talk else None
+
+    def step_bytes(self, rows):
+        return sum(w.w.numel() * w.w.element_size() for w in (self.w_in, self.w_o))
+
+    def step_flops(self, rows):
+        return 2 * rows * (self.w_in.w.numel() + self.w_o.w.numel())
+
+    def mixing_flops(self, past, new):
+        """Scores once, weighted values once for every key-value head (the mixing is done behind the sum over keys)."""
+        keys = sum(min(past + t + 1, self.window) if self.window else past + t + 1 for t in range(new)) if self.window \
+            else new * past + new * (new + 1) // 2
+        return 2 * self.H * (self.dk + self.dv * (self.G if self.talk is not None else 1)) * keys
+
+    def forward(self, x, step, view):
+        """The whole mixer, its output bias added."""
+        out = self.rt.linear(self.attend(self.project(x, step, view), step, view), self.w_o)
+        return out.add_(self.output_bias.to(out.dtype))
+
+    def forward_unbiased(self, x, step, view):
+        """(result without the output projection's bias, possibly as partial planes; that bias in float32): for a
+        block that adds both to the residual stream itself."""
+        return self.output(self.attend(self.project(x, step, view), step, view)), self.output_bias
+
+    def project(self, x, step, view):
+        """q (and k, v) of the step's tokens with their biases, q and k turned by position, k and v stored."""
+        rt = self.rt
+        if view.need.head_dim != self.dk or view.need.v_dim != self.dv or view.need.n_kv_heads != self.G:
+            raise ValueError("the cache's pages do not have this layer's head counts and sizes")
+        qkv = rt.linear(x, self.w_in)
+        if self.rot and step.max_position >= self.position.n_positions:
+            raise ValueError(f"position {step.max_position} is past the rotary table of {self.position.n_positions}")
+        store = not self.borrows
+        if store != bool(view.store):
+            raise ValueError("a layer with key and value projections keeps its own pages, a borrowing layer reads another's")
+        rt.ops.qkv_prepare(qkv, self.bias_in, self.position.table if self.rot else None, self.rot, step,
+                           view.block_table(step), view.k, view.v, view.page_size, self.H, self.G, self.dk, self.dv,
+                           write_kv=store)
+        return qkv
+
+    def attend(self, qkv, step, view):
+        rt = self.rt
+        out = torch.empty(qkv.shape[0], self.H * self.dv, dtype=rt.dtype, device=qkv.device)
+        return rt.ops.sink_attn(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
+                                view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window)
+
+    def output(self, attended):
+        return self.rt.linear(attended, self.w_o, partials=True)
