@@ -294,9 +294,12 @@ def test_a_place_with_several_needs_gets_a_view_for_each():
     assert c.bytes_read(40) == (3 * 40 + 32) * 2 * (2 * 8) * c.views[1].k.element_size()
     c.close(s)
     assert c.open() == s and float(c.views[0][1].tensor[s].abs().sum()) == 0.0
-    with pytest.raises(CacheError, match="several needs"):
-        make([kv, (kv, StateNeed((2,)))], [None, 0])
+    # a place with several needs reads another's keys and values with its KVNeed and keeps its states; one lends its own
+    c2 = make([kv, (kv, StateNeed((2,)))], [None, 0])
+    assert c2.views[1][0].k.data_ptr() == c2.views[0].k.data_ptr() and not c2.views[1][0].store
+    c3 = make([(kv, StateNeed((2,))), kv], [None, 0])
+    assert c3.views[1].k.data_ptr() == c3.views[0][0].k.data_ptr() and len(c3.groups[0].places) == 1
     with pytest.raises(CacheError, match="keeps keys and values of its own"):
-        make([(kv, StateNeed((2,))), kv], [None, 0])                    # a place with several needs lends none
+        make([(StateNeed((2,)), None), kv], [None, 0])                  # nothing to lend
     with pytest.raises(CacheError, match="a need is"):
         make([(kv, "keys")])
