@@ -321,6 +321,30 @@ def fuvirax_config(width, ff, heads, layers, vocab):
                 layers=[kinds[i % 3] for i in range(layers)])
 
 
+def digasun_config(width, ff, heads, layers, vocab):
+    """Gated linear attention, attention with a window of 1,024 keys, and attention that borrows the layer before's
+    keys and values, in turn; heads of 128 lanes in groups of four; the dense feed-forward of the first kind of layer
+    has the Llama's inner size (8,192: the same three matrices), the experts of the other two together with their
+    shared expert as many weights (8 of 768, 2 chosen, and 2,048 shared)."""
+    dense = dict(kind="dense", ff=8192, limit=7.0)
+    moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=768), shared=dict(ff=2048))
+    att = dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=1024),
+               rot=dict(base=500000.0, dims=128))
+    made = []
+    for i in range(layers):
+        if i % 3 == 0:
+            made.append(dict(type="gla", mlp=dense, mixer=dict(heads=heads, dim=128, vdim=128, tau=16.0, decay_rank=64)))
+        elif i % 3 == 1:
+            made.append(dict(type="attention", mlp=moe, mixer=dict(att)))
+        else:
+            made.append(dict(type="attention", mlp=moe, mixer=dict(att, kv_from=i - 1)))
+    return dict(architecture="Digasun", vocab=vocab, width=width, canon=dict(taps=4), embedding=dict(scale=1.0),
+                norm=dict(eps=1e-6), token_side=dict(dim=64), layers=made)
+
+
+DESIGNS = {"fuvirax": fuvirax_config, "digasun": digasun_config}
+
+
 def mixer_rates(engine, batch, context, prefill_tokens):
     """The mixing kernels of every kind of mixer in the engine alone (no projections), at a decode step of `batch`
     sequences that hold `context` tokens and at a prompt of `prefill_tokens`: time, and the rate against the limit
@@ -330,10 +354,14 @@ def mixer_rates(engine, batch, context, prefill_tokens):
     out, seen = {}, {}
     for i, pl in enumerate(model.plan.order):
         m = model.blocks[pl.layer].mixer
+        if getattr(m, "borrows", False):
+            continue
         seen.setdefault(type(m).__name__, (model.blocks[pl.layer], engine.cache.views[i]))
     width = model.plan.width
 
     def mixer_view(block, view):
+        if hasattr(block, "_mixer_view"):
+            return block._mixer_view(view)
         return block._views(view)[1] if hasattr(block, "_views") else view
 
     def run(kind, block, view, step, x, tag, nbytes=None, flops=None):
@@ -346,6 +374,12 @@ def mixer_rates(engine, batch, context, prefill_tokens):
             mid, mix = m.project(x), m.scan
         elif kind == "ChannelDelta":
             mid, mix = m.project(x, step, v), m.scan
+        elif kind == "SinkAttention":
+            if m.borrows:        # the lending layer's kernel is the same one
+                return
+            mid, mix = m.project(x, step, v), m.attend
+        elif kind == "GatedLinearAttention":
+            mid, mix = m.project(x), m.scan
         else:
             return
         mix(mid, step, v)          # once outside the recording
@@ -361,7 +395,7 @@ def mixer_rates(engine, batch, context, prefill_tokens):
             out[key + "_gbs"] = round(nbytes / sec / 1e9, 1)
             out[key + "_frac"] = round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4)
         if flops is not None:
-            peak = MFMA_PEAK["bf16"] if kind in ("Attention", "LatentAttention") else MFMA_PEAK["fp32"]
+            peak = MFMA_PEAK["bf16"] if kind in ("Attention", "LatentAttention", "SinkAttention") else MFMA_PEAK["fp32"]
             out[key + "_tflops"] = round(flops / sec / 1e12, 2)
             out[key + "_frac"] = round(flops / sec / peak, 4)
 
@@ -371,7 +405,8 @@ def mixer_rates(engine, batch, context, prefill_tokens):
         kv = [v for v in views if isinstance(v, KVView)]
         if kv:
             n = kv[0].need
-            return batch * context * (n.n_kv_heads * n.head_dim + n.v_heads * n.v_dim) * kv[0].k.element_size()
+            keys = min(context, n.window) if n.window > 0 else context
+            return batch * keys * (n.n_kv_heads * n.head_dim + n.v_heads * n.v_dim) * kv[0].k.element_size()
         return 2 * batch * max(v.tensor[0].numel() * v.tensor.element_size() for v in views)
 
     slots = [engine.open() for _ in range(batch)]
@@ -396,14 +431,14 @@ def mixer_rates(engine, batch, context, prefill_tokens):
 
 
 def run_design(args):
-    """--design fuvirax: prompt and decode throughput of the design at sizes that resemble a real model's layers
+    """--design fuvirax | digasun: prompt and decode throughput of the design at sizes that resemble a real model's layers
     (random weights), beside the Llama of equal size, and the mixing kernels of both alone against their limits."""
     import torch
     from burn_lm_amd.config.presets import preset
     from burn_lm_amd.engine.loading import random_engine
     from burn_lm_amd.sampling.sampler import Sampler
-    if args.design != "fuvirax":
-        print(f"bench.py: no design named {args.design!r}; known: fuvirax")
+    if args.design not in DESIGNS:
+        print(f"bench.py: no design named {args.design!r}; known: {', '.join(DESIGNS)}")
         sys.exit(2)
     layers = args.layers or 6
     record = {"metric": "design_throughput", "design": args.design, "dtype": args.dtype, "data": "synthetic", "n_gpus": 1,
@@ -413,7 +448,7 @@ def run_design(args):
         size = DESIGN_SIZES[name]
         base = preset(size["llama"])
         base["num_hidden_layers"] = layers
-        configs = {"fuvirax": fuvirax_config(size["width"], size["ff"], size["heads"], layers, base["vocab_size"]),
+        configs = {args.design: DESIGNS[args.design](size["width"], size["ff"], size["heads"], layers, base["vocab_size"]),
                    "llama": base}
         entry = {}
         for model, config in configs.items():
@@ -497,7 +532,7 @@ def main():
                          "launched kernel by kernel on a cache that is filled without a prompt step; prints its time and "
                          "no JSON line, and says on stderr where it is")
     ap.add_argument("--design", default=None, metavar="NAME",
-                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax) at model-like "
+                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax, digasun) at model-like "
                          "layer sizes beside the Llama of equal size, with the mixing kernels alone (--layers, default 6; "
                          "--sizes 1b-like,3b-like)")
     ap.add_argument("--sizes", default=None, help="with --design: which of its sizes, with commas between them")

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 30
+ABI_VERSION = 31
 _lib = None
 _lock = threading.Lock()
 
@@ -39,6 +39,10 @@ _SIGNATURES = {
                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_sink_attn_mfma_supported": [_c_int, _c_int],
+    "blm_sink_attn_mfma": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                           _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                           _c_int, _c_float, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_sink_attn": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                       _c_void_p],
@@ -1244,4 +1248,47 @@ def sink_attn(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, 
     _call("blm_sink_attn", q.data_ptr(), q.stride(0), out.data_ptr(), _code(q), A.data_ptr(), _ptr(sinks), _ptr(mix),
           step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1],
           kcache.data_ptr(), vcache.data_ptr(), page_size, T, H, G, dk, dv, float(scale), int(window), _stream())
+    return out
+
+
+def sink_attn_mfma_supported(dtype, dk, dv, page_size=64):
+    return dtype == torch.bfloat16 and page_size == 64 and bool(library().blm_sink_attn_mfma_supported(int(dk), int(dv)))
+
+
+def sink_attn_mfma_max_splits(n_seqs, max_new, H, G, dv, mixed):
+    """Most pieces the matrix-core form can cut a tile's pages into for a step of this shape (its partial results
+    live in the fixed workspace of latent_attn_init)."""
+    cols = n_seqs * G * ((max_new * (H // G) + 15) // 16) * 16
+    return max(1, min(64, LATENT_SCRATCH_FLOATS // (cols * ((G if mixed else 1) * dv + 2))))
+
+
+def sink_attn_mfma(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, H, G, dk, dv, scale, window, n_splits=1):
+    """sink_attn on the matrix cores: bfloat16 queries, pages (64 keys) and output; the same arguments, and n_splits:
+    into how many pieces every tile's pages are cut (a second kernel adds them up)."""
+    _gpu(q, out, sinks, mix, block_table, kcache, vcache)
+    T = q.shape[0]
+    _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
+    if q.stride(1) != 1 or not (q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16):
+        raise KernelError("sink_attn_mfma: queries, pages and output in bfloat16; rows contiguous")
+    if tuple(out.shape) != (T, H * dv) or tuple(kcache.shape[1:]) != (G, page_size, dk) \
+            or tuple(vcache.shape) != (kcache.shape[0], G, dv, page_size) or T != step.n_tokens \
+            or block_table.shape[0] < step.n_seqs or step.cu_seqlens.numel() < step.n_seqs + 1:
+        raise KernelError(f"sink_attn_mfma: shapes do not fit: out {tuple(out.shape)}, pages {tuple(kcache.shape)} / {tuple(vcache.shape)}")
+    if sinks is not None:
+        _f32("sinks", sinks, H)
+    if mix is not None:
+        _f32("mix", mix, H * H)
+    n_out = G if mix is not None else 1
+    A = torch.empty(T, H, n_out, dv, dtype=torch.float32, device=q.device)
+    part_o = part_ml = None
+    if n_splits > 1:
+        if n_splits > sink_attn_mfma_max_splits(step.n_seqs, step.max_new, H, G, dv, mix is not None):
+            raise KernelError("sink_attn_mfma: more pieces than the workspace holds (see sink_attn_mfma_max_splits)")
+        cols = step.n_seqs * G * ((step.max_new * (H // G) + 15) // 16) * 16
+        buf = latent_attn_init(q.device)
+        part_o, part_ml = buf[: cols * n_splits * n_out * dv], buf[cols * n_splits * n_out * dv: cols * n_splits * (n_out * dv + 2)]
+    _call("blm_sink_attn_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), A.data_ptr(), _ptr(sinks), _ptr(mix),
+          step.token_seq.data_ptr(), step.cu_seqlens.data_ptr(), step.lens_after.data_ptr(), block_table.data_ptr(),
+          block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(), page_size, step.n_seqs, step.max_new, T, H, G, dk, dv,
+          float(scale), int(window), int(n_splits), _ptr(part_o), _ptr(part_ml), _stream())
     return out

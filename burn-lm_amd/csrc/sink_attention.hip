@@ -200,9 +200,13 @@ __global__ void sink_attn_kernel(const TA* __restrict__ q, int ldq, float* __res
 
 // out[t][h][d] = sum_g mix[h][g] * A[t][g][c(h)][d]  (mix null: A has one slot per head and is only converted)
 template <typename TA>
-__global__ void talk_mix_kernel(const float* __restrict__ A, const float* __restrict__ mix, TA* __restrict__ out, int H,
-                                int G, int dv) {
+__global__ void talk_mix_kernel(const float* __restrict__ A, const float* __restrict__ mix, TA* __restrict__ out,
+                                const int* __restrict__ token_seq, int H, int G, int dv) {
   const int t = blockIdx.x;
+  if (token_seq[t] < 0) {      // a padding token: nobody wrote its rows of A
+    for (int e = threadIdx.x; e < H * dv; e += blockDim.x) out[(size_t)t * H * dv + e] = from_float<TA>(0.f);
+    return;
+  }
   const int n_slots = mix ? G : 1;
   const float* a = A + (size_t)t * H * n_slots * dv;
   for (int e = threadIdx.x; e < H * dv; e += blockDim.x) {
@@ -217,6 +221,17 @@ __global__ void talk_mix_kernel(const float* __restrict__ A, const float* __rest
     }
     out[(size_t)t * H * dv + e] = from_float<TA>(v);
   }
+}
+
+static int launch_talk_mix(const float* A, const float* mix, void* out, int dtype, const int* token_seq, int T, int H, int G,
+                           int dv, hipStream_t stream) {
+  const int threads = H * dv >= 1024 ? 512 : 256;
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(T), dim3(threads), 0, stream, A, mix, (float*)out, token_seq, H, G, dv);
+  else
+    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(T), dim3(threads), 0, stream, A, mix, (bf16*)out, token_seq, H, G, dv);
+  BLM_LAUNCH_CHECK("talk_mix");
+  return 0;
 }
 
 extern "C" int blm_sink_attn(const void* q, int ldq, void* out, int dtype, float* A, const float* sinks, const float* mix,
@@ -254,11 +269,312 @@ extern "C" int blm_sink_attn(const void* q, int ldq, void* out, int dtype, float
 #undef SA_PICK
 #undef SA_CASE
   BLM_LAUNCH_CHECK("sink_attn");
-  const int threads = H * dv >= 1024 ? 512 : 256;
-  if (dtype == BLM_F32)
-    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(T), dim3(threads), 0, stream, A, mix, (float*)out, H, G, dv);
-  else
-    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(T), dim3(threads), 0, stream, A, mix, (bf16*)out, H, G, dv);
-  BLM_LAUNCH_CHECK("talk_mix");
-  return 0;
+  return launch_talk_mix(A, mix, out, dtype, token_seq, T, H, G, dv, stream);
+}
+
+// ---------------------------------------------------------------------------------------
+// The same function on the matrix cores (bfloat16, pages of 64 keys).  A wavefront's 16 query columns are
+// 16 (token, head) pairs of one sequence whose heads share a key-value head, so that one tile of keys serves
+// them all.  Per page:
+//   S^T = K Q^T      A operand = 16 keys x 32 lanes of a key row per instruction, B = Q^T; lane (kg, c) gets the
+//                    scores of column c for keys kg*4 .. kg*4+3 of each 16-key tile
+//   O_g^T += V_g^T P^T  for every key-value head g of the batch: A = 16 value lanes x 32 keys from the transposed
+//                    value pages, B = the probabilities the lane has just computed (the keys of a page are dealt
+//                    to the four score tiles so that the eight keys a lane supplies are neighbours there)
+// The running maximum starts at the sink's logit and the sum at one (in the first piece of a cut range).  Fragments
+// come straight from global memory; the four wavefronts of a block are neighbouring tiles, which read the same
+// pages at the same time.  With n_splits > 1 the pages of a tile are cut into pieces that a second kernel adds up.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 sa_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float sa_f32x4;
+
+__device__ __forceinline__ constexpr int sa_key_of(int t, int i) { return (t >> 1) * 32 + (i >> 2) * 8 + (t & 1) * 4 + (i & 3); }
+
+__device__ __forceinline__ uint4 sa_keep_first(uint4 v, int n) {      // the first n (0..8) bf16 of 16 bytes, zeros behind
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int left = n - 2 * i;
+    w[i] = left >= 2 ? w[i] : (left == 1 ? (w[i] & 0xffffu) : 0u);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+#define SAM_WAVES 4
+#define SAM_MAX_PIECES 64
+template <int KS, int DT, int GB>
+__global__ void __launch_bounds__(SAM_WAVES* BLM_WAVE)
+    sink_attn_mfma_kernel(const bf16* __restrict__ q, int ldq, float* __restrict__ A, const float* __restrict__ sinks,
+                          const int* __restrict__ cu_seqlens, const int* __restrict__ lens_after,
+                          const int* __restrict__ block_table, int table_width, const bf16* __restrict__ kcache,
+                          const bf16* __restrict__ vcache, int B, int H, int G, int dk, int dv, int tiles_per_seq,
+                          float scale2, int window, int all_groups, int n_splits, float* __restrict__ part_o,
+                          float* __restrict__ part_ml) {
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const long long tile_id = (long long)blockIdx.x * SAM_WAVES + wave;      // over sequences x key-value heads x tiles
+  const int tile = (int)(tile_id % tiles_per_seq);
+  const int kvh = (int)((tile_id / tiles_per_seq) % G);
+  const long long b = tile_id / ((long long)tiles_per_seq * G);
+  if (b >= B) return;
+  const int split = blockIdx.y;
+  const int Hg = H / G;
+  const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
+  const int n_cols = n_new * Hg;
+  if (tile * 16 >= n_cols) return;                                         // also a padding sequence
+  const int after = lens_after[b];
+  const int past = after - n_new;
+  const int idx = tile * 16 + c;
+  const bool valid = idx < n_cols;
+  const int tok = valid ? idx / Hg : 0, head = kvh * Hg + (valid ? idx - tok * Hg : 0);
+  const int qpos = valid ? past + tok : -1;
+  const int min_qpos = past + (tile * 16) / Hg;
+  const int max_qpos = past + min(tile * 16 + 15, n_cols - 1) / Hg;
+  const int max_key = after - 1;
+  const int first_key = (window > 0 && min_qpos - window + 1 > 0) ? min_qpos - window + 1 : 0;
+  const int p_lo = first_key / 64, p_hi = max_qpos / 64;
+  const int per = (p_hi - p_lo + 1 + n_splits - 1) / n_splits;
+  const int p_begin = p_lo + split * per, p_end = min(p_hi + 1, p_begin + per);
+  const int* bt = block_table + (size_t)b * table_width;
+  const int n_out = all_groups ? G : 1;
+  const int g0 = all_groups ? blockIdx.z * GB : kvh;
+
+  uint4 qf[KS];
+  {
+    const bf16* qrow = q + (size_t)(t_first + tok) * ldq + (size_t)head * dk;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + kg * 8;
+      qf[ks] = (valid && d < dk) ? *reinterpret_cast<const uint4*>(qrow + d) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  const bool sunk = valid && sinks != nullptr && split == 0;
+  float m = sunk ? sinks[head] * 1.4426950408889634f : -INFINITY;
+  sa_f32x4 l = sunk ? sa_f32x4{1.f, 1.f, 1.f, 1.f} : sa_f32x4{0.f, 0.f, 0.f, 0.f};
+  sa_f32x4 o[GB][DT];
+#pragma unroll
+  for (int gi = 0; gi < GB; ++gi)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[gi][dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int pi = p_begin; pi < p_end; ++pi) {
+    const int page = bt[pi];
+    const int key0 = pi * 64;
+    const bf16* kp = kcache + ((size_t)page * G + kvh) * 64 * dk;
+    float s[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bf16* krow = kp + (size_t)sa_key_of(t, c) * dk;
+      uint4 kf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + kg * 8;
+        kf[ks] = d < dk ? *reinterpret_cast<const uint4*>(krow + d) : make_uint4(0u, 0u, 0u, 0u);
+      }
+      sa_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sa_bf16x8, kf[ks]),
+                                                      __builtin_bit_cast(sa_bf16x8, qf[ks]), acc, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kj = key0 + sa_key_of(t, kg * 4 + r);
+        const bool seen = kj <= qpos && (window <= 0 || kj > qpos - window);
+        s[t][r] = seen ? acc[r] : -INFINITY;      // whatever the places past the data hold, it is replaced here
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[t][r]);
+    mx = rows_max(mx);
+    const float m_new = fmaxf(m, mx * scale2);
+    const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        s[t][r] = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
+    if (__any(m != m_new)) {
+#pragma unroll
+      for (int gi = 0; gi < GB; ++gi)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[gi][dt][r] *= corr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) l[r] *= corr;
+    }
+    m = m_new;
+    const bool tail = key0 + 63 > max_key;       // the page holds places past the data: 0 * garbage must stay 0
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 pf;
+      pf.x = f32x2_to_bf16x2_bits(s[2 * h][0], s[2 * h][1]);
+      pf.y = f32x2_to_bf16x2_bits(s[2 * h][2], s[2 * h][3]);
+      pf.z = f32x2_to_bf16x2_bits(s[2 * h + 1][0], s[2 * h + 1][1]);
+      pf.w = f32x2_to_bf16x2_bits(s[2 * h + 1][2], s[2 * h + 1][3]);
+      // the softmax's denominator: a row of ones in place of V^T sums the rounded probabilities of every column
+      l = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          __builtin_bit_cast(sa_bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u)),
+          __builtin_bit_cast(sa_bf16x8, pf), l, 0, 0, 0);
+      const int keep = max_key - (key0 + h * 32 + kg * 8) + 1;
+#pragma unroll
+      for (int gi = 0; gi < GB; ++gi) {
+        const int cc = g0 + gi;
+        if (cc < G) {
+          const bf16* vp = vcache + ((size_t)page * G + cc) * dv * 64;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const int row = dt * 16 + c;
+            uint4 va = row < dv ? *reinterpret_cast<const uint4*>(vp + (size_t)row * 64 + h * 32 + kg * 8) : make_uint4(0u, 0u, 0u, 0u);
+            if (tail) va = sa_keep_first(va, keep);
+            o[gi][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sa_bf16x8, va),
+                                                                __builtin_bit_cast(sa_bf16x8, pf), o[gi][dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (n_splits == 1) {
+    if (valid) {
+      const float inv = 1.0f / l[0];
+      float* arow = A + ((size_t)(t_first + tok) * H + head) * n_out * dv;
+#pragma unroll
+      for (int gi = 0; gi < GB; ++gi) {
+        const int cc = g0 + gi;
+        if (cc < G) {
+          float* og = arow + (size_t)(all_groups ? cc : 0) * dv;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int d = dt * 16 + kg * 4 + r;
+              if (d < dv) og[d] = o[gi][dt][r] * inv;
+            }
+        }
+      }
+    }
+    return;
+  }
+  // leave this piece: per column its maximum, sum and unnormalised results; sink_merge_kernel adds the pieces up
+  const size_t gcol = (size_t)tile_id * 16 + c;
+  float* po = part_o + (gcol * n_splits + split) * n_out * dv;
+#pragma unroll
+  for (int gi = 0; gi < GB; ++gi) {
+    const int cc = g0 + gi;
+    if (cc < G) {
+      float* og = po + (size_t)(all_groups ? cc : 0) * dv;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int d = dt * 16 + kg * 4 + r;
+          if (d < dv) og[d] = o[gi][dt][r];
+        }
+    }
+  }
+  if (kg == 0 && blockIdx.z == 0) {
+    part_ml[(gcol * n_splits + split) * 2] = m;
+    part_ml[(gcol * n_splits + split) * 2 + 1] = l[0];
+  }
+}
+
+// The pieces of a cut range added up, one block per column: maxima in base 2.  A piece that saw nothing and holds
+// no sink has sum 0, maximum -infinity and results of zeros, and gets weight 0.
+__global__ void __launch_bounds__(256)
+    sink_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, float* __restrict__ A,
+                      const int* __restrict__ cu_seqlens, int H, int G, int n_out, int dv, int tiles_per_seq, int n_splits) {
+  __shared__ float wgt[SAM_MAX_PIECES];
+  __shared__ float inv_sum;
+  const size_t gcol = blockIdx.x;
+  const int c = (int)(gcol & 15);
+  const long long tile_id = (long long)(gcol >> 4);
+  const int tile = (int)(tile_id % tiles_per_seq);
+  const int kvh = (int)((tile_id / tiles_per_seq) % G);
+  const long long b = tile_id / ((long long)tiles_per_seq * G);
+  const int Hg = H / G;
+  const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
+  const int idx = tile * 16 + c;
+  if (idx >= n_new * Hg) return;
+  const int tok = idx / Hg, head = kvh * Hg + idx - tok * Hg;
+  const float* ml = part_ml + gcol * n_splits * 2;
+  if (threadIdx.x < BLM_WAVE) {          // n_splits <= 64: one lane per piece
+    const bool has = (int)threadIdx.x < n_splits;
+    const float ms = has ? ml[threadIdx.x * 2] : -INFINITY, ls = has ? ml[threadIdx.x * 2 + 1] : 0.f;
+    const float M = wave_max(ls != 0.f ? ms : -INFINITY);
+    const float w = ls != 0.f ? __builtin_amdgcn_exp2f(ms - M) : 0.f;
+    const float L = wave_sum(ls * w);
+    if (has) wgt[threadIdx.x] = w;
+    if (threadIdx.x == 0) inv_sum = 1.0f / L;
+  }
+  __syncthreads();
+  const int n = n_out * dv;
+  const float* po = part_o + gcol * n_splits * n;
+  float* arow = A + ((size_t)(t_first + tok) * H + head) * n;
+  for (int d = threadIdx.x; d < n; d += blockDim.x) {
+    float acc = 0.f;
+    for (int p = 0; p < n_splits; ++p) acc = fmaf(wgt[p], po[(size_t)p * n + d], acc);
+    arow[d] = acc * inv_sum;
+  }
+}
+
+extern "C" int blm_sink_attn_mfma_supported(int dk, int dv) {
+  return (dk % 8 == 0 && dk >= 8 && dk <= 128 && dv >= 1 && dv <= 128) ? 1 : 0;
+}
+
+// q: bfloat16 rows of ldq elements (queries at column 0, already rotated); out bfloat16 [T][H * dv]; A: float
+// [T][H][G or 1][dv] workspace; pages in bfloat16, 64 keys each.  B sequences of at most max_new tokens.  Workspace for
+// n_splits > 1: part_o (B * G * tiles * 16 * n_splits * (G or 1) * dv floats), part_ml (B * G * tiles * 16 * n_splits * 2),
+// with tiles = ceil(max_new * (H / G) / 16).
+extern "C" int blm_sink_attn_mfma(const void* q, int ldq, void* out, float* A, const float* sinks, const float* mix,
+                                  const int* token_seq, const int* cu_seqlens, const int* lens_after, const int* block_table,
+                                  int table_width, const void* kcache, const void* vcache, int page_size, int B, int max_new,
+                                  int T, int H, int G, int dk, int dv, float scale, int window, int n_splits, float* part_o,
+                                  float* part_ml, hipStream_t stream) {
+  BLM_REQUIRE(B > 0 && max_new > 0 && T > 0 && H > 0 && G > 0 && H % G == 0, "sink_attn_mfma: bad sizes B=%d H=%d G=%d", B, H, G);
+  BLM_REQUIRE(page_size == 64 && table_width > 0 && window >= 0, "sink_attn_mfma: pages of 64 keys");
+  BLM_REQUIRE(blm_sink_attn_mfma_supported(dk, dv), "sink_attn_mfma: head sizes %d / %d are not among those it takes", dk, dv);
+  BLM_REQUIRE(scale > 0.f && ldq % 8 == 0 && ldq >= H * dk && ((size_t)q & 15) == 0, "sink_attn_mfma: a positive scale and query rows that start at multiples of 16 bytes");
+  BLM_REQUIRE(n_splits >= 1 && n_splits <= SAM_MAX_PIECES && (n_splits == 1 || (part_o && part_ml)),
+              "sink_attn_mfma: %d pieces (1 to %d, with their workspace)", n_splits, SAM_MAX_PIECES);
+  const int all_groups = mix ? 1 : 0;
+  const int gb = !all_groups ? 1 : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+  const long long tiles = ((long long)max_new * (H / G) + 15) / 16;
+  const long long waves = (long long)B * G * tiles;
+  BLM_REQUIRE(waves < 2147483647LL, "sink_attn_mfma: too many tiles");
+  dim3 grid((unsigned)((waves + SAM_WAVES - 1) / SAM_WAVES), (unsigned)n_splits, (unsigned)(all_groups ? (G + gb - 1) / gb : 1));
+  const float scale2 = scale * 1.4426950408889634f;
+  const int ks = dk <= 64 ? 2 : 4;
+  const int dt = dv <= 32 ? 2 : (dv <= 48 ? 3 : (dv <= 64 ? 4 : 8));
+#define SAM_CASE(KS, DT, GB)                                                                                              \
+  hipLaunchKernelGGL((sink_attn_mfma_kernel<KS, DT, GB>), grid, dim3(SAM_WAVES * BLM_WAVE), 0, stream, (const bf16*)q, ldq, A, \
+                     sinks, cu_seqlens, lens_after, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache, B, H, \
+                     G, dk, dv, (int)tiles, scale2, window, all_groups, n_splits, part_o, part_ml)
+#define SAM_GB(KS, DT)                  \
+  do {                                  \
+    if (gb == 4) SAM_CASE(KS, DT, 4);   \
+    else if (gb == 2) SAM_CASE(KS, DT, 2); \
+    else SAM_CASE(KS, DT, 1);           \
+  } while (0)
+#define SAM_DT(KS)                      \
+  do {                                  \
+    if (dt == 2) SAM_GB(KS, 2);         \
+    else if (dt == 3) SAM_GB(KS, 3);    \
+    else if (dt == 4) SAM_GB(KS, 4);    \
+    else SAM_GB(KS, 8);                 \
+  } while (0)
+  if (ks == 2) SAM_DT(2);
+  else SAM_DT(4);
+#undef SAM_DT
+#undef SAM_GB
+#undef SAM_CASE
+  BLM_LAUNCH_CHECK("sink_attn_mfma");
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(sink_merge_kernel, dim3((unsigned)(waves * 16)), dim3(256), 0, stream, part_o, part_ml, A, cu_seqlens, H,
+                       G, all_groups ? G : 1, dv, (int)tiles, n_splits);
+    BLM_LAUNCH_CHECK("sink_merge");
+  }
+  return launch_talk_mix(A, mix, out, BLM_BF16, token_seq, T, H, G, dv, stream);
 }

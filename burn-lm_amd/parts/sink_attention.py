@@ -11,6 +11,8 @@ that an earlier layer keeps, with queries, window, sink and mixing of its own.  
 are float32 in every mode."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .base import KVNeed, Mixer, TensorSpec
@@ -69,6 +71,10 @@ class SinkAttention(Mixer):
         self.bias_in = torch.cat([tensors[n[r + "_bias"]].float() for r in roles]).contiguous()
         self.w_o = rt.weight(tensors[n["o"]])
         self.output_bias = tensors[n["o_bias"]].float().contiguous()
+        self.on_matrix_cores = rt.ops.sink_attn_mfma_supported(rt.dtype, self.dk, self.dv) and self.scale > 0 \
+            and os.environ.get("BURN_LM_AMD_SINK_ATTENTION") != "generic"
+        if self.on_matrix_cores:
+            rt.ops.latent_attn_init(rt.device)     # the pieces' workspace, before any step is recorded
         self.sinks = tensors[n["sink"]].float().contiguous() if sink else None
         self.talk = tensors[n["talk"]].float().contiguous() if talk else None
 
@@ -111,8 +117,25 @@ class SinkAttention(Mixer):
         return qkv
 
     def attend(self, qkv, step, view):
+        """Every token's queries over its sequence's visible keys -> [tokens, heads * vdim].  bfloat16 with pages of
+        64 keys and head sizes the matrix-core kernel takes: that kernel, its pages cut into pieces when a step
+        brings so few tiles (decoding) that they would leave most of the chip idle; else the generic kernel."""
         rt = self.rt
         out = torch.empty(qkv.shape[0], self.H * self.dv, dtype=rt.dtype, device=qkv.device)
+        if self.on_matrix_cores and view.page_size == 64 and qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 \
+                and hasattr(step, "lens_after"):
+            n_splits = 1
+            if step.max_new == 1:
+                span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
+                pages = (span + view.page_size - 1) // view.page_size
+                batches = -(-self.G // 4) if self.talk is not None else 1
+                tiles = step.n_seqs * self.G * -(-(self.H // self.G) // 16) * batches
+                n_splits = max(1, min(pages // 2, (2 * rt.compute_units) // max(1, tiles),
+                                      rt.ops.sink_attn_mfma_max_splits(step.n_seqs, 1, self.H, self.G, self.dv,
+                                                                       self.talk is not None)))
+            return rt.ops.sink_attn_mfma(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
+                                         view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window,
+                                         n_splits=n_splits)
         return rt.ops.sink_attn(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
                                 view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window)
 
