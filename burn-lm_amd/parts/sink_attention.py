@@ -130,7 +130,7 @@ class SinkAttention(Mixer):
                 pages = (span + view.page_size - 1) // view.page_size
                 batches = -(-self.G // 4) if self.talk is not None else 1
                 tiles = step.n_seqs * self.G * -(-(self.H // self.G) // 16) * batches
-                n_splits = max(1, min(pages // 2, (2 * rt.compute_units) // max(1, tiles),
+                n_splits = max(1, min(pages, (4 * rt.compute_units) // max(1, tiles),
                                       rt.ops.sink_attn_mfma_max_splits(step.n_seqs, 1, self.H, self.G, self.dv,
                                                                        self.talk is not None)))
             return rt.ops.sink_attn_mfma(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
