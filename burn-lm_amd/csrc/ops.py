@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 31
+ABI_VERSION = 32
 _lib = None
 _lock = threading.Lock()
 
@@ -36,13 +36,14 @@ _SIGNATURES = {
     "blm_moe_route": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
     "blm_moe_gate": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_gla_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_float, _c_void_p, _c_void_p,
-                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_sink_attn_mfma_supported": [_c_int, _c_int],
     "blm_sink_attn_mfma": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                            _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                           _c_int, _c_float, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+                           _c_int, _c_float, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_sink_attn": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                       _c_void_p],
@@ -1180,10 +1181,25 @@ def moe_gate(gate_up, weights, out, n_experts, expert_inner):
     return out
 
 
-def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, step, H, dk, dv):
+def gla_segments(step, H, dv, compute_units=256):
+    """(segments, tokens per segment) into which gla_scan cuts the sequences of a step: prompts are walked by several
+    wavefronts at once, each over a stretch of at least 64 tokens (a multiple of 8), as many as give every compute
+    unit about thirty-two wavefronts; steps of few tokens per sequence are not cut."""
+    if step.n_tokens <= 4 * step.n_seqs or step.max_new < 128 or dv > 256:
+        return 1, 0
+    walkers = step.n_seqs * H * ((dv + 3) // 4)
+    n_seg = max(1, min(step.max_new // 64, (32 * compute_units) // max(1, walkers)))
+    if n_seg == 1:
+        return 1, 0
+    seg_len = (-(-step.max_new // n_seg) + 7) // 8 * 8
+    return -(-step.max_new // seg_len), seg_len
+
+
+def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, step, H, dk, dv, segments=None):
     """Gated linear attention over proj [T, >= 2 H dk + 2 H dv]: queries, keys, values, output-gate logits;
     decay_in [T, H dk]: the decays' logits before their bias.  state float32 [slots, H, dk, dv] is read and left
-    updated; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in proj's dtype."""
+    updated; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in proj's dtype.  segments: (count, tokens each) as
+    gla_segments gives them (the default), or (1, 0) for one walk per sequence."""
     _gpu(proj, decay_in, decay_bias, norm_w, state, o_raw, out)
     T = proj.shape[0]
     _f32("o_raw", o_raw, T * H * dv); _f32("decay_bias", decay_bias, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
@@ -1192,9 +1208,18 @@ def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, st
     if proj.stride(1) != 1 or out.dtype != proj.dtype or decay_in.dtype != proj.dtype or tuple(out.shape) != (T, H * dv) \
             or tuple(decay_in.shape) != (T, H * dk) or tuple(state.shape[1:]) != (H, dk, dv):
         raise KernelError("gla_scan: shapes do not fit")
+    n_seg, seg_len = segments if segments is not None else gla_segments(step, H, dv)
+    seg_end = seg_start = seg_decay = q_tilde = None
+    if n_seg > 1:
+        B = step.n_seqs
+        seg_end = torch.empty(B, n_seg, H, dk, dv, dtype=torch.float32, device=proj.device)
+        seg_start = torch.empty_like(seg_end)
+        seg_decay = torch.empty(B, n_seg, H, dk, dtype=torch.float32, device=proj.device)
+        q_tilde = torch.empty(T, H, dk, dtype=torch.float32, device=proj.device)
     _call("blm_gla_scan", proj.data_ptr(), _code(proj), proj.stride(0), decay_in.data_ptr(), decay_bias.data_ptr(), float(tau),
           norm_w.data_ptr(), float(eps), state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(),
-          step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs, H, dk, dv, _stream())
+          step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs, H, dk, dv, step.max_new, n_seg, seg_len,
+          _ptr(seg_end), _ptr(seg_start), _ptr(seg_decay), _ptr(q_tilde), _stream())
     return out
 
 
@@ -1262,9 +1287,11 @@ def sink_attn_mfma_max_splits(n_seqs, max_new, H, G, dv, mixed):
     return max(1, min(64, LATENT_SCRATCH_FLOATS // (cols * ((G if mixed else 1) * dv + 2))))
 
 
-def sink_attn_mfma(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, H, G, dk, dv, scale, window, n_splits=1):
+def sink_attn_mfma(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, H, G, dk, dv, scale, window, n_splits=1,
+                   group_batch=0):
     """sink_attn on the matrix cores: bfloat16 queries, pages (64 keys) and output; the same arguments, and n_splits:
-    into how many pieces every tile's pages are cut (a second kernel adds them up)."""
+    into how many pieces every tile's pages are cut (a second kernel adds them up); group_batch: 0, or the most
+    key-value heads a wavefront accumulates at a time (fewer: more wavefronts, each with less to wait for)."""
     _gpu(q, out, sinks, mix, block_table, kcache, vcache)
     T = q.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
@@ -1290,5 +1317,5 @@ def sink_attn_mfma(q, out, sinks, mix, step, block_table, kcache, vcache, page_s
     _call("blm_sink_attn_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), A.data_ptr(), _ptr(sinks), _ptr(mix),
           step.token_seq.data_ptr(), step.cu_seqlens.data_ptr(), step.lens_after.data_ptr(), block_table.data_ptr(),
           block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(), page_size, step.n_seqs, step.max_new, T, H, G, dk, dv,
-          float(scale), int(window), int(n_splits), _ptr(part_o), _ptr(part_ml), _stream())
+          float(scale), int(window), int(n_splits), int(group_batch), _ptr(part_o), _ptr(part_ml), _stream())
     return out

@@ -26,14 +26,15 @@ __global__ void input_conv_kernel(const float* __restrict__ n, const float* __re
                                   const int* __restrict__ seq_slots, int D) {
   const int t = blockIdx.x;
   const int b = token_seq[t];
+  const int c_first = blockIdx.y * blockDim.x + threadIdx.x, c_step = gridDim.y * blockDim.x;
   if (b < 0) {
-    for (int c = threadIdx.x; c < D; c += blockDim.x)
+    for (int c = c_first; c < D; c += c_step)
       for (int r = 0; r < readers; ++r) ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(0.f);
     return;
   }
   const int start = cu_seqlens[b], slot = seq_slots[b];
   const int off = t - start;
-  for (int c = threadIdx.x; c < D; c += blockDim.x) {
+  for (int c = c_first; c < D; c += c_step) {
     float x[PB_MAX_TAPS];
 #pragma unroll
     for (int k = 0; k < PB_MAX_TAPS; ++k) {
@@ -92,12 +93,14 @@ extern "C" int blm_input_conv(const float* n, float* hist, const float* w0, cons
     rd.w[r] = weights[r];
     rd.out[r] = outs[r];
   }
-  const int threads = D >= 1024 ? 512 : (D >= 256 ? 256 : 128);
+  // few tokens (decoding): a token's channels over several blocks, so that more than a handful of compute units work
+  const int threads = 256;
+  const unsigned pieces = T >= 512 ? 1u : (unsigned)((D + threads - 1) / threads);
   if (out_dtype == BLM_F32)
-    hipLaunchKernelGGL(input_conv_kernel<float>, dim3(T), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+    hipLaunchKernelGGL(input_conv_kernel<float>, dim3(T, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
                        cu_seqlens, seq_slots, D);
   else if (out_dtype == BLM_BF16)
-    hipLaunchKernelGGL(input_conv_kernel<bf16>, dim3(T), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+    hipLaunchKernelGGL(input_conv_kernel<bf16>, dim3(T, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
                        cu_seqlens, seq_slots, D);
   else
     return blm_fail("input_conv: unsupported dtype %d", out_dtype);
@@ -260,6 +263,29 @@ __global__ void clamped_glu_kernel(const TA* __restrict__ gate_up, TA* __restric
   }
 }
 
+// eight bfloat16 at a time (I a multiple of 8, rows that start at multiples of 16 bytes)
+__device__ __forceinline__ float pb_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float pb_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__global__ void clamped_glu8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, long long n8, int I8, float limit,
+                                    float alpha) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n8; e += stride) {
+    const long long t = e / I8;
+    const int i = (int)(e - t * I8);
+    const uint4 g4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + i) * 8);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + I8 + i) * 8);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g0 = fminf(pb_lo(gw[k]), limit), g1 = fminf(pb_hi(gw[k]), limit);
+      const float u0 = fminf(fmaxf(pb_lo(uw[k]), -limit), limit), u1 = fminf(fmaxf(pb_hi(uw[k]), -limit), limit);
+      r[k] = f32x2_to_bf16x2_bits(g0 * pb_sigmoid(alpha * g0) * (u0 + 1.0f), g1 * pb_sigmoid(alpha * g1) * (u1 + 1.0f));
+    }
+    *reinterpret_cast<uint4*>(out + (size_t)e * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+  }
+}
+
 extern "C" int blm_clamped_glu(const void* gate_up, void* out, int dtype, int T, int I, float limit, float alpha,
                                hipStream_t stream) {
   BLM_REQUIRE(T > 0 && I > 0 && limit > 0.f, "clamped_glu: bad sizes T=%d I=%d limit=%g", T, I, (double)limit);
@@ -267,7 +293,11 @@ extern "C" int blm_clamped_glu(const void* gate_up, void* out, int dtype, int T,
   const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, (float*)out, n, I, limit, alpha);
-  else if (dtype == BLM_BF16)
+  else if (dtype == BLM_BF16 && I % 8 == 0 && ((size_t)gate_up & 15) == 0 && ((size_t)out & 15) == 0) {
+    const long long n8 = n / 8;
+    const unsigned b8 = (unsigned)((n8 + 255) / 256 < 65535 ? (n8 + 255) / 256 : 65535);
+    hipLaunchKernelGGL(clamped_glu8_kernel, dim3(b8), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, n8, I / 8, limit, alpha);
+  } else if (dtype == BLM_BF16)
     hipLaunchKernelGGL(clamped_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, n, I, limit, alpha);
   else
     return blm_fail("clamped_glu: unsupported dtype %d", dtype);
@@ -339,6 +369,30 @@ __global__ void moe_gate_kernel(const TA* __restrict__ gate_up, const float* __r
   }
 }
 
+// eight bfloat16 at a time (the experts' inner sizes and I multiples of 8: eight neighbours belong to one expert)
+__global__ void moe_gate8_kernel(const bf16* __restrict__ gate_up, const float* __restrict__ weights, bf16* __restrict__ out,
+                                 long long n8, int I8, int E, int ffe8) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n8; e += stride) {
+    const long long t = e / I8;
+    const int i = (int)(e - t * I8);
+    const int ex = i / ffe8 < E ? i / ffe8 : E;
+    const float w = weights[(size_t)t * (E + 1) + ex];
+    uint32_t r[4] = {0u, 0u, 0u, 0u};
+    if (w != 0.f) {
+      const uint4 g4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + i) * 8);
+      const uint4 u4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + I8 + i) * 8);
+      const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float g0 = pb_lo(gw[k]), g1 = pb_hi(gw[k]);
+        r[k] = f32x2_to_bf16x2_bits(g0 * pb_sigmoid(g0) * pb_lo(uw[k]) * w, g1 * pb_sigmoid(g1) * pb_hi(uw[k]) * w);
+      }
+    }
+    *reinterpret_cast<uint4*>(out + (size_t)e * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+  }
+}
+
 extern "C" int blm_moe_gate(const void* gate_up, const float* weights, void* out, int dtype, int T, int I, int E, int ffe,
                             hipStream_t stream) {
   BLM_REQUIRE(T > 0 && E > 0 && ffe > 0 && I >= E * ffe, "moe_gate: bad sizes T=%d I=%d experts=%d of %d", T, I, E, ffe);
@@ -346,7 +400,11 @@ extern "C" int blm_moe_gate(const void* gate_up, const float* weights, void* out
   const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(moe_gate_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, weights, (float*)out, n, I, E, ffe);
-  else if (dtype == BLM_BF16)
+  else if (dtype == BLM_BF16 && I % 8 == 0 && ffe % 8 == 0 && ((size_t)gate_up & 15) == 0 && ((size_t)out & 15) == 0) {
+    const long long n8 = n / 8;
+    const unsigned b8 = (unsigned)((n8 + 255) / 256 < 65535 ? (n8 + 255) / 256 : 65535);
+    hipLaunchKernelGGL(moe_gate8_kernel, dim3(b8), dim3(256), 0, stream, (const bf16*)gate_up, weights, (bf16*)out, n8, I / 8, E, ffe / 8);
+  } else if (dtype == BLM_BF16)
     hipLaunchKernelGGL(moe_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)gate_up, weights, (bf16*)out, n, I, E, ffe);
   else
     return blm_fail("moe_gate: unsupported dtype %d", dtype);

@@ -214,8 +214,8 @@ struct ScanLaunch {
   dim3 grid, block;
   size_t smem;
 };
-static ScanLaunch scan_launch(int rows, int lpc, int vectors, long long items) {
-  const size_t per_wave = (size_t)SCAN_CHUNK * (vectors * lpc * (rows + 4) + (vectors - 1) * SCAN_COLS) * sizeof(float);
+static ScanLaunch scan_launch(int rows, int lpc, int vectors, long long items, int chunk = SCAN_CHUNK) {
+  const size_t per_wave = (size_t)chunk * (vectors * lpc * (rows + 4) + (vectors - 1) * SCAN_COLS) * sizeof(float);
   int waves = (int)((64 * 1024) / per_wave);
   waves = waves > SCAN_WAVES ? SCAN_WAVES : (waves < 1 ? 1 : waves);
   ScanLaunch sl;
@@ -573,20 +573,32 @@ __global__ void gla_gates_kernel(const TA* __restrict__ decay_in, const float* _
     gates[e] = expf(-blm_softplus(-(to_float(decay_in[e]) + bias[e % HK])) * inv_tau);
 }
 
-template <typename TA, int ROWS, int LPC>
+// With SEG a sequence's tokens are cut into n_seg segments of seg_len tokens that different wavefronts walk at the
+// same time: the first from the sequence's state, the others from zero.  The recurrence is linear in the state, so
+//   S_t = (prod of the segment's decays up to t) S_start + (what the walk from zero gives),
+//   o_t = (q_t * that product)^T S_start + (the walk's o_t):
+// a segment leaves its end state, the product of all its decays and, per token, the query times the running product;
+// gla_carry_kernel then passes the true start states from segment to segment (and leaves the sequence's state), and
+// gla_apply_kernel adds the first term to the results.  Decays are at most one, so the products cannot overflow.
+template <typename TA, int ROWS, int LPC, bool SEG, int CH>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     gla_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates, float q_scale,
                     float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
-                    const int* __restrict__ seq_slots, int H, int dk, int dv, int col_groups, long long n_items) {
+                    const int* __restrict__ seq_slots, int H, int dk, int dv, int col_groups, long long n_items,
+                    int n_seg, int seg_len, float* __restrict__ seg_end, float* __restrict__ seg_decay,
+                    float* __restrict__ q_tilde) {
   extern __shared__ __attribute__((aligned(16))) float scan_sm[];     // per wavefront: [chunk][decay | k | q][vec], [chunk][16 values]
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const long long item = (long long)blockIdx.x * (blockDim.x / BLM_WAVE) + wave;
   if (item >= n_items) return;
   const int cg = (int)(item % col_groups);
   const int h = (int)((item / col_groups) % H);
-  const int b = (int)(item / ((long long)col_groups * H));
+  const int seg = SEG ? (int)((item / ((long long)col_groups * H)) % n_seg) : 0;
+  const int b = (int)(item / ((long long)col_groups * H * (SEG ? n_seg : 1)));
   const int slot = seq_slots[b];
-  const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+  const int seq_end = cu_seqlens[b + 1];
+  const int t0 = cu_seqlens[b] + seg * (SEG ? seg_len : 0);
+  const int t1 = SEG ? min(seq_end, t0 + seg_len) : seq_end;
   if (slot < 0 || t1 <= t0) return;
   constexpr int COLS = BLM_WAVE / LPC;
   const int g = LPC == 4 ? lane >> 4 : lane & 15, cl = LPC == 4 ? lane & 15 : lane >> 4;
@@ -594,20 +606,22 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   const bool own = col < dv;
   constexpr int dkp = ROWS * LPC;
   constexpr int vec = LPC * (ROWS + 4);
-  float* base = scan_sm + (size_t)wave * SCAN_CHUNK * (3 * vec + 2 * SCAN_COLS);
-  float* v_sm = base + SCAN_CHUNK * 3 * vec;
+  float* base = scan_sm + (size_t)wave * CH * (3 * vec + 2 * SCAN_COLS);
+  float* v_sm = base + CH * 3 * vec;
   float* S_g = state + (((size_t)slot * H + h) * dk) * dv;
-  float S[ROWS];
+  float S[ROWS], D[SEG ? ROWS : 1];
 #pragma unroll
   for (int r = 0; r < ROWS; ++r) {
     const int i = g * ROWS + r;
-    S[r] = (own && i < dk) ? S_g[(size_t)i * dv + col] : 0.f;
+    S[r] = (own && i < dk && seg == 0) ? S_g[(size_t)i * dv + col] : 0.f;
+    if (SEG) D[r] = 1.f;
   }
+  const bool writes_rows = SEG && cl == 0 && cg == 0;      // one column's lanes write what belongs to the rows alone
   constexpr int PER = (dkp + BLM_WAVE - 1) / BLM_WAVE;
-  float raw_d[SCAN_CHUNK][PER], raw_k[SCAN_CHUNK][PER], raw_q[SCAN_CHUNK][PER], v_in[SCAN_CHUNK];
+  float raw_d[CH][PER], raw_k[CH][PER], raw_q[CH][PER], v_in[CH];
   auto fetch = [&](int tc) {
 #pragma unroll
-    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+    for (int tt = 0; tt < CH; ++tt) {
       if (tc + tt < t1) {
         const int t = tc + tt;
         const TA* row = proj + (size_t)t * ld;
@@ -626,10 +640,10 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     }
   };
   fetch(t0);
-  for (int tc = t0; tc < t1; tc += SCAN_CHUNK) {
-    const int n = min(SCAN_CHUNK, t1 - tc);
+  for (int tc = t0; tc < t1; tc += CH) {
+    const int n = min(CH, t1 - tc);
 #pragma unroll
-    for (int tt = 0; tt < SCAN_CHUNK; ++tt) {
+    for (int tt = 0; tt < CH; ++tt) {
       if (tt < n) {
         if (g == 0) v_sm[tt * 2 * SCAN_COLS + cl] = v_in[tt];
 #pragma unroll
@@ -644,7 +658,7 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
         }
       }
     }
-    if (tc + SCAN_CHUNK < t1) fetch(tc + SCAN_CHUNK);     // the next chunk's inputs travel while this one runs
+    if (tc + CH < t1) fetch(tc + CH);     // the next chunk's inputs travel while this one runs
     __builtin_amdgcn_wave_barrier();
 #pragma unroll 1
     for (int tt = 0; tt < n; ++tt) {
@@ -661,6 +675,11 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
         for (int e = 0; e < 4; ++e) {
           S[r + e] = fmaf(d[e], S[r + e], kk[e] * vv);
           o = fmaf(S[r + e], q[e], o);
+          if (SEG) {
+            D[r + e] *= d[e];
+            if (writes_rows && seg > 0 && g * ROWS + r + e < dk)
+              q_tilde[((size_t)(tc + tt) * H + h) * dk + g * ROWS + r + e] = q[e] * D[r + e];
+          }
         }
       }
       o = column_sum<LPC>(o);
@@ -668,23 +687,113 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
     }
     __builtin_amdgcn_wave_barrier();
   }
+  float* S_out = SEG ? seg_end + ((((size_t)b * n_seg + seg) * H + h) * dk) * dv : S_g;
   if (own) {
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
       const int i = g * ROWS + r;
-      if (i < dk) S_g[(size_t)i * dv + col] = S[r];
+      if (i < dk) S_out[(size_t)i * dv + col] = S[r];
+    }
+  }
+  if (writes_rows) {
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+      const int i = g * ROWS + r;
+      if (i < dk) seg_decay[(((size_t)b * n_seg + seg) * H + h) * dk + i] = D[SEG ? r : 0];
     }
   }
 }
 
+// From segment to segment: start[s + 1] = decay[s] * start[s] + end[s], with start[1] = end[0] (the first segment
+// walked from the sequence's own state); what comes out behind the last segment is the sequence's state.
+__global__ void gla_carry_kernel(const float* __restrict__ seg_end, const float* __restrict__ seg_decay,
+                                 float* __restrict__ seg_start, float* __restrict__ state, const int* __restrict__ cu_seqlens,
+                                 const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg, int seg_len) {
+  const int b = blockIdx.y;
+  const int slot = seq_slots[b];
+  const int n_new = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || n_new <= 0) return;
+  const int ns = (n_new + seg_len - 1) / seg_len;
+  const size_t per = (size_t)H * dk * dv;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < per; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t row = e / dv;      // h * dk + i
+    float S = seg_end[((size_t)b * n_seg) * per + e];
+    for (int sgm = 1; sgm < ns; ++sgm) {
+      seg_start[((size_t)b * n_seg + sgm) * per + e] = S;
+      S = fmaf(seg_decay[((size_t)b * n_seg + sgm) * H * dk + row], S, seg_end[((size_t)b * n_seg + sgm) * per + e]);
+    }
+    state[(size_t)slot * per + e] = S;
+  }
+}
+
+// o_raw[t][h][:] += q_tilde[t][h][:]^T start[segment of t][h] for the tokens of every segment but a sequence's first;
+// one wavefront per (eight tokens of one segment, head), a lane per value channel (and its neighbours 64 apart).
+#define GLA_APPLY_TOKENS 8
+#define GLA_APPLY_CPL 4
+__global__ void __launch_bounds__(BLM_WAVE)
+    gla_apply_kernel(const float* __restrict__ q_tilde, const float* __restrict__ seg_start, float* __restrict__ o_raw,
+                     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg,
+                     int seg_len, int tiles_per_seq) {
+  extern __shared__ float qt[];      // [8][dk]
+  const int b = blockIdx.x / tiles_per_seq, tile = blockIdx.x - b * tiles_per_seq;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - first;
+  const int off = tile * GLA_APPLY_TOKENS;
+  if (seq_slots[b] < 0 || off >= n_new) return;
+  const int seg = off / seg_len;      // seg_len is a multiple of eight: the tile lies in one segment
+  if (seg == 0) return;
+  const int n = min(GLA_APPLY_TOKENS, n_new - off);
+  for (int e = lane; e < n * dk; e += BLM_WAVE) {
+    const int tt = e / dk, i = e - tt * dk;
+    qt[tt * dk + i] = q_tilde[((size_t)(first + off + tt) * H + h) * dk + i];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const float* Sp = seg_start + ((((size_t)b * n_seg + seg) * H + h) * dk) * dv;
+  float acc[GLA_APPLY_TOKENS][GLA_APPLY_CPL];
+#pragma unroll
+  for (int tt = 0; tt < GLA_APPLY_TOKENS; ++tt)
+#pragma unroll
+    for (int c = 0; c < GLA_APPLY_CPL; ++c) acc[tt][c] = 0.f;
+  for (int i = 0; i < dk; ++i) {
+    float sv[GLA_APPLY_CPL];
+#pragma unroll
+    for (int c = 0; c < GLA_APPLY_CPL; ++c) {
+      const int j = lane + c * BLM_WAVE;
+      sv[c] = j < dv ? Sp[(size_t)i * dv + j] : 0.f;
+    }
+#pragma unroll
+    for (int tt = 0; tt < GLA_APPLY_TOKENS; ++tt) {
+      const float qv = tt < n ? qt[tt * dk + i] : 0.f;
+#pragma unroll
+      for (int c = 0; c < GLA_APPLY_CPL; ++c) acc[tt][c] = fmaf(qv, sv[c], acc[tt][c]);
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < GLA_APPLY_TOKENS; ++tt) {
+    if (tt < n) {
+#pragma unroll
+      for (int c = 0; c < GLA_APPLY_CPL; ++c) {
+        const int j = lane + c * BLM_WAVE;
+        if (j < dv) o_raw[((size_t)(first + off + tt) * H + h) * dv + j] += acc[tt][c];
+      }
+    }
+  }
+}
+
+// n_seg > 1 (only where the sequences bring many tokens each, T > 4 B): seg_len a multiple of 8 with n_seg * seg_len >= the
+// most tokens of a sequence; seg_end and seg_start [B][n_seg][H][dk][dv], seg_decay [B][n_seg][H][dk], q_tilde [T][H][dk].
 extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* decay_in, const float* decay_bias, float tau,
                             const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
-                            const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv,
+                            const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv, int max_new,
+                            int n_seg, int seg_len, float* seg_end, float* seg_start, float* seg_decay, float* q_tilde,
                             hipStream_t stream) {
   BLM_REQUIRE(T > 0 && B > 0 && H > 0 && tau > 0.f, "gla_scan: bad sizes T=%d B=%d H=%d tau=%g", T, B, H, (double)tau);
   BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "gla_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(ld >= 2 * H * dk + 2 * H * dv, "gla_scan: rows of %d are too short", ld);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "gla_scan: unsupported dtype %d", dtype);
+  BLM_REQUIRE(n_seg >= 1 && (n_seg == 1 || (T > 4 * B && seg_len >= 8 && seg_len % 8 == 0 && (long long)n_seg * seg_len >= max_new &&
+                                            dv <= BLM_WAVE * GLA_APPLY_CPL && seg_end && seg_start && seg_decay && q_tilde)),
+              "gla_scan: %d segments of %d tokens do not fit this step", n_seg, seg_len);
   {
     const long long n = (long long)T * H * dk;
     const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
@@ -695,19 +804,46 @@ extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* dec
     BLM_LAUNCH_CHECK("gla_gates");
   }
   const float q_scale = 1.0f / sqrtf((float)dk);
-#define BLM_GLA(ROWS, LPC)                                                                                                \
+#define BLM_GLA_RUN(ROWS, LPC, SEG, NSEG, CH)                                                                             \
   const int col_groups = (dv + 64 / LPC - 1) / (64 / LPC);                                                                \
-  const long long items = (long long)B * H * col_groups;                                                                  \
-  const ScanLaunch sl = scan_launch(ROWS, LPC, 3, items);                                                                 \
+  const long long items = (long long)B * NSEG * H * col_groups;                                                           \
+  const ScanLaunch sl = scan_launch(ROWS, LPC, 3, items, CH);                                                             \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((gla_scan_kernel<float, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
-                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items);                       \
+    hipLaunchKernelGGL((gla_scan_kernel<float, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
+                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items, n_seg, seg_len, seg_end, \
+                       seg_decay, q_tilde);                                                                               \
   else                                                                                                                    \
-    hipLaunchKernelGGL((gla_scan_kernel<bf16, ROWS, LPC>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
-                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items)
-  BLM_SCAN_PICK(BLM_GLA);
+    hipLaunchKernelGGL((gla_scan_kernel<bf16, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
+                       q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items, n_seg, seg_len, seg_end, \
+                       seg_decay, q_tilde)
+  // segments: many wavefronts at once, each waiting for its own chain of dependent instructions; chunks of four tokens halve
+  // a wavefront's shared memory, so that twice as many of them share a compute unit
+#define BLM_GLA(ROWS, LPC) BLM_GLA_RUN(ROWS, LPC, false, 1, SCAN_CHUNK)
+#define BLM_GLA_SEG(ROWS) BLM_GLA_RUN(ROWS, 16, true, n_seg, 4)
+  if (n_seg > 1) {
+    const int rows = (dk + 15) / 16;
+    if (rows <= 4) { BLM_GLA_SEG(4); }
+    else if (rows <= 8) { BLM_GLA_SEG(8); }
+    else { BLM_GLA_SEG(16); }
+  } else {
+    BLM_SCAN_PICK(BLM_GLA);
+  }
+#undef BLM_GLA_SEG
 #undef BLM_GLA
+#undef BLM_GLA_RUN
   BLM_LAUNCH_CHECK("gla_scan");
+  if (n_seg > 1) {
+    const size_t per = (size_t)H * dk * dv;
+    const unsigned cb = (unsigned)((per + 255) / 256 < 1024 ? (per + 255) / 256 : 1024);
+    hipLaunchKernelGGL(gla_carry_kernel, dim3(cb, B), dim3(256), 0, stream, seg_end, seg_decay, seg_start, state, cu_seqlens,
+                       seq_slots, H, dk, dv, n_seg, seg_len);
+    BLM_LAUNCH_CHECK("gla_carry");
+    const int tiles_per_seq = (max_new + GLA_APPLY_TOKENS - 1) / GLA_APPLY_TOKENS;
+    hipLaunchKernelGGL(gla_apply_kernel, dim3((unsigned)(B * tiles_per_seq), H), dim3(BLM_WAVE),
+                       (size_t)GLA_APPLY_TOKENS * dk * sizeof(float), stream, q_tilde, seg_start, o_raw, cu_seqlens, seq_slots, H,
+                       dk, dv, n_seg, seg_len, tiles_per_seq);
+    BLM_LAUNCH_CHECK("gla_apply");
+  }
   const char* gate = (const char*)proj + (size_t)(2 * H * dk + H * dv) * (dtype == BLM_F32 ? 4 : 2);
   return launch_head_norm(o_raw, norm_w, gate, ld, 2, H, out, dtype, (long long)T * H, dv, eps, stream);
 }

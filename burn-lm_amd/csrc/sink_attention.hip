@@ -198,38 +198,39 @@ __global__ void sink_attn_kernel(const TA* __restrict__ q, int ldq, float* __res
   }
 }
 
-// out[t][h][d] = sum_g mix[h][g] * A[t][g][c(h)][d]  (mix null: A has one slot per head and is only converted)
+// out[t][h][d] = sum_g mix[h][g] * A[t][g][c(h)][d]  (mix null: A has one slot per head and is only converted); a block
+// per (token, head)
 template <typename TA>
 __global__ void talk_mix_kernel(const float* __restrict__ A, const float* __restrict__ mix, TA* __restrict__ out,
                                 const int* __restrict__ token_seq, int H, int G, int dv) {
-  const int t = blockIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y;
+  TA* o = out + ((size_t)t * H + h) * dv;
   if (token_seq[t] < 0) {      // a padding token: nobody wrote its rows of A
-    for (int e = threadIdx.x; e < H * dv; e += blockDim.x) out[(size_t)t * H * dv + e] = from_float<TA>(0.f);
+    for (int d = threadIdx.x; d < dv; d += blockDim.x) o[d] = from_float<TA>(0.f);
     return;
   }
   const int n_slots = mix ? G : 1;
   const float* a = A + (size_t)t * H * n_slots * dv;
-  for (int e = threadIdx.x; e < H * dv; e += blockDim.x) {
-    const int h = e / dv, d = e - h * dv;
+  const int c = h / (H / G);
+  for (int d = threadIdx.x; d < dv; d += blockDim.x) {
     float v;
     if (mix) {
-      const int c = h / (H / G);
       v = 0.f;
       for (int g = 0; g < H; ++g) v = fmaf(mix[h * H + g], a[((size_t)g * G + c) * dv + d], v);
     } else {
       v = a[(size_t)h * dv + d];
     }
-    out[(size_t)t * H * dv + e] = from_float<TA>(v);
+    o[d] = from_float<TA>(v);
   }
 }
 
 static int launch_talk_mix(const float* A, const float* mix, void* out, int dtype, const int* token_seq, int T, int H, int G,
                            int dv, hipStream_t stream) {
-  const int threads = H * dv >= 1024 ? 512 : 256;
+  const int threads = dv > 64 ? 128 : 64;
   if (dtype == BLM_F32)
-    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(T), dim3(threads), 0, stream, A, mix, (float*)out, token_seq, H, G, dv);
+    hipLaunchKernelGGL(talk_mix_kernel<float>, dim3(T, H), dim3(threads), 0, stream, A, mix, (float*)out, token_seq, H, G, dv);
   else
-    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(T), dim3(threads), 0, stream, A, mix, (bf16*)out, token_seq, H, G, dv);
+    hipLaunchKernelGGL(talk_mix_kernel<bf16>, dim3(T, H), dim3(threads), 0, stream, A, mix, (bf16*)out, token_seq, H, G, dv);
   BLM_LAUNCH_CHECK("talk_mix");
   return 0;
 }
@@ -527,12 +528,12 @@ extern "C" int blm_sink_attn_mfma_supported(int dk, int dv) {
 // q: bfloat16 rows of ldq elements (queries at column 0, already rotated); out bfloat16 [T][H * dv]; A: float
 // [T][H][G or 1][dv] workspace; pages in bfloat16, 64 keys each.  B sequences of at most max_new tokens.  Workspace for
 // n_splits > 1: part_o (B * G * tiles * 16 * n_splits * (G or 1) * dv floats), part_ml (B * G * tiles * 16 * n_splits * 2),
-// with tiles = ceil(max_new * (H / G) / 16).
+// with tiles = ceil(max_new * (H / G) / 16).  group_batch: 0, or the most key-value heads a wavefront accumulates (1, 2, 4).
 extern "C" int blm_sink_attn_mfma(const void* q, int ldq, void* out, float* A, const float* sinks, const float* mix,
                                   const int* token_seq, const int* cu_seqlens, const int* lens_after, const int* block_table,
                                   int table_width, const void* kcache, const void* vcache, int page_size, int B, int max_new,
-                                  int T, int H, int G, int dk, int dv, float scale, int window, int n_splits, float* part_o,
-                                  float* part_ml, hipStream_t stream) {
+                                  int T, int H, int G, int dk, int dv, float scale, int window, int n_splits, int group_batch,
+                                  float* part_o, float* part_ml, hipStream_t stream) {
   BLM_REQUIRE(B > 0 && max_new > 0 && T > 0 && H > 0 && G > 0 && H % G == 0, "sink_attn_mfma: bad sizes B=%d H=%d G=%d", B, H, G);
   BLM_REQUIRE(page_size == 64 && table_width > 0 && window >= 0, "sink_attn_mfma: pages of 64 keys");
   BLM_REQUIRE(blm_sink_attn_mfma_supported(dk, dv), "sink_attn_mfma: head sizes %d / %d are not among those it takes", dk, dv);
@@ -540,7 +541,10 @@ extern "C" int blm_sink_attn_mfma(const void* q, int ldq, void* out, float* A, c
   BLM_REQUIRE(n_splits >= 1 && n_splits <= SAM_MAX_PIECES && (n_splits == 1 || (part_o && part_ml)),
               "sink_attn_mfma: %d pieces (1 to %d, with their workspace)", n_splits, SAM_MAX_PIECES);
   const int all_groups = mix ? 1 : 0;
-  const int gb = !all_groups ? 1 : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+  // key-value heads per wavefront: up to four share one walk over the keys; fewer (group_batch) spreads a step of few
+  // tiles over more wavefronts, each of which then waits for fewer fragments
+  int gb = !all_groups ? 1 : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+  if (group_batch >= 1 && group_batch < gb) gb = group_batch >= 2 ? 2 : 1;
   const long long tiles = ((long long)max_new * (H / G) + 15) / 16;
   const long long waves = (long long)B * G * tiles;
   BLM_REQUIRE(waves < 2147483647LL, "sink_attn_mfma: too many tiles");

@@ -124,18 +124,19 @@ class SinkAttention(Mixer):
         out = torch.empty(qkv.shape[0], self.H * self.dv, dtype=rt.dtype, device=qkv.device)
         if self.on_matrix_cores and view.page_size == 64 and qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 \
                 and hasattr(step, "lens_after"):
-            n_splits = 1
+            n_splits, group_batch = 1, 0
             if step.max_new == 1:
                 span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
                 pages = (span + view.page_size - 1) // view.page_size
-                batches = -(-self.G // 4) if self.talk is not None else 1
+                group_batch = int(os.environ.get("BURN_LM_AMD_SINK_GROUP_BATCH", "1"))
+                batches = -(-self.G // max(1, min(4, group_batch or 4))) if self.talk is not None else 1
                 tiles = step.n_seqs * self.G * -(-(self.H // self.G) // 16) * batches
                 n_splits = max(1, min(pages, (4 * rt.compute_units) // max(1, tiles),
                                       rt.ops.sink_attn_mfma_max_splits(step.n_seqs, 1, self.H, self.G, self.dv,
                                                                        self.talk is not None)))
             return rt.ops.sink_attn_mfma(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
                                          view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window,
-                                         n_splits=n_splits)
+                                         n_splits=n_splits, group_batch=group_batch)
         return rt.ops.sink_attn(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
                                 view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window)
 

@@ -403,7 +403,7 @@ def _attend(form, *args):
     from burn_lm_amd.csrc import ops
     if form == "generic":
         return ops.sink_attn(*args)
-    return ops.sink_attn_mfma(*args, n_splits=1 if form == "matrix" else 3)
+    return ops.sink_attn_mfma(*args, n_splits=1 if form == "matrix" else 3, group_batch=0 if form == "matrix" else 1)
 
 
 FORMS = [("generic", torch.float32), ("generic", torch.bfloat16), ("matrix", torch.bfloat16), ("matrix_pieces", torch.bfloat16)]
