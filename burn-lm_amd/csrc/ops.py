@@ -99,6 +99,7 @@ _SIGNATURES = {
     "blm_gemm_rows": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_void_p],
     "blm_attn_paged_init": [],
+    "blm_sink_attn_mfma_init": [],
     "blm_gemm_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_void_p],
     "blm_gemv_mfma_group_limit": [_c_int],
@@ -1276,6 +1277,20 @@ def sink_attn(q, out, sinks, mix, step, block_table, kcache, vcache, page_size, 
     return out
 
 
+_sam_ready = set()
+
+
+def sink_attn_mfma_init(device=None):
+    """Once per device, outside any stream capture, before the first sink_attn_mfma of a prompt (the form that stages
+    pages takes more shared memory than a kernel gets without asking)."""
+    index = torch.device(device or "cuda").index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _sam_ready:
+        with torch.cuda.device(index):
+            _call("blm_sink_attn_mfma_init")
+        _sam_ready.add(index)
+
+
 def sink_attn_mfma_supported(dtype, dk, dv, page_size=64):
     return dtype == torch.bfloat16 and page_size == 64 and bool(library().blm_sink_attn_mfma_supported(int(dk), int(dv)))
 
@@ -1293,6 +1308,7 @@ def sink_attn_mfma(q, out, sinks, mix, step, block_table, kcache, vcache, page_s
     into how many pieces every tile's pages are cut (a second kernel adds them up); group_batch: 0, or the most
     key-value heads a wavefront accumulates at a time (fewer: more wavefronts, each with less to wait for)."""
     _gpu(q, out, sinks, mix, block_table, kcache, vcache)
+    sink_attn_mfma_init(q.device)
     T = q.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache); _i32("block_table", block_table)
     if q.stride(1) != 1 or not (q.dtype == out.dtype == kcache.dtype == vcache.dtype == torch.bfloat16):

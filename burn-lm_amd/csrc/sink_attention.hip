@@ -482,6 +482,202 @@ __global__ void __launch_bounds__(SAM_WAVES* BLM_WAVE)
   }
 }
 
+// The same for steps of many tokens (prompts): the four wavefronts of a block are four neighbouring tiles of one
+// sequence and key-value head, which see nearly the same pages; the block brings every page once, keys and the values
+// of the batch's key-value heads, into shared memory (16 bytes per thread and load, whole pages in order; rows padded
+// by 16 bytes so that the fragment reads of 16 rows fall on different banks), and the wavefronts take their fragments
+// from there.  Without it every wavefront fetches every fragment itself, and the second-level cache's rate bounds
+// the kernel.  A wavefront skips the pages outside its own tile's range but meets the others at every page.
+template <int KS, int DT, int GB>
+__global__ void __launch_bounds__(SAM_WAVES* BLM_WAVE)
+    sink_attn_mfma_staged_kernel(const bf16* __restrict__ q, int ldq, float* __restrict__ A, const float* __restrict__ sinks,
+                                 const int* __restrict__ cu_seqlens, const int* __restrict__ lens_after,
+                                 const int* __restrict__ block_table, int table_width, const bf16* __restrict__ kcache,
+                                 const bf16* __restrict__ vcache, int B, int H, int G, int dk, int dv, int blocks_per_seq,
+                                 float scale2, int window, int all_groups) {
+  extern __shared__ __attribute__((aligned(16))) bf16 sam_sm[];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const int blk = blockIdx.x % blocks_per_seq;
+  const int kvh = (blockIdx.x / blocks_per_seq) % G;
+  const int b = blockIdx.x / (blocks_per_seq * G);
+  const int Hg = H / G;
+  const int t_first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t_first;
+  const int n_cols = n_new * Hg;
+  if (blk * 64 >= n_cols) return;                                          // the whole block: also a padding sequence
+  const int after = lens_after[b];
+  const int past = after - n_new;
+  const int tile = blk * SAM_WAVES + wave;
+  const bool active = tile * 16 < n_cols;
+  const int idx = tile * 16 + c;
+  const bool valid = active && idx < n_cols;
+  const int tok = valid ? idx / Hg : 0, head = kvh * Hg + (valid ? idx - tok * Hg : 0);
+  const int qpos = valid ? past + tok : -1;
+  const int max_key = after - 1;
+  auto first_page = [&](int col) { const int p = past + col / Hg; return (window > 0 && p - window + 1 > 0) ? (p - window + 1) / 64 : 0; };
+  auto last_page = [&](int col) { return (past + min(col, n_cols - 1) / Hg) / 64; };
+  const int my_lo = active ? first_page(tile * 16) : 1, my_hi = active ? last_page(tile * 16 + 15) : 0;
+  const int blk_lo = first_page(blk * 64), blk_hi = last_page(blk * 64 + 63);
+  const int* bt = block_table + (size_t)b * table_width;
+  const int n_out = all_groups ? G : 1;
+  const int g0 = all_groups ? blockIdx.z * GB : kvh;
+  const int krs = dk + 8, vrs = 64 + 8;                                    // padded rows, in elements
+  bf16* k_sm = sam_sm;                                                     // [64][krs]
+  bf16* v_sm = sam_sm + 64 * krs;                                          // [GB][dv][vrs]
+
+  uint4 qf[KS];
+  {
+    const bf16* qrow = q + (size_t)(t_first + tok) * ldq + (size_t)head * dk;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + kg * 8;
+      qf[ks] = (valid && d < dk) ? *reinterpret_cast<const uint4*>(qrow + d) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+  const bool sunk = valid && sinks != nullptr;
+  float m = sunk ? sinks[head] * 1.4426950408889634f : -INFINITY;
+  sa_f32x4 l = sunk ? sa_f32x4{1.f, 1.f, 1.f, 1.f} : sa_f32x4{0.f, 0.f, 0.f, 0.f};
+  sa_f32x4 o[GB][DT];
+#pragma unroll
+  for (int gi = 0; gi < GB; ++gi)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[gi][dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int k_pieces = dk / 8;                                             // 16-byte pieces per key row
+
+  // a page travels in two steps: from memory into registers while the page before is worked on, from there into
+  // shared memory once nobody reads that page any more
+  constexpr int KP = 4, VP = 4;            // 16-byte pieces per thread: keys (64 rows of up to 128 lanes), values per key-value head
+  uint4 k_in[KP], v_in[GB][VP];
+#define SAM_FETCH(PI)                                                                                     \
+  {                                                                                                       \
+    const int page_ = bt[PI];                                                                             \
+    const bf16* kp_ = kcache + ((size_t)page_ * G + kvh) * 64 * dk;                                       \
+    _Pragma("unroll") for (int u = 0; u < KP; ++u) {                                                      \
+      const int e = threadIdx.x + u * SAM_WAVES * BLM_WAVE;                                               \
+      k_in[u] = e < 64 * k_pieces ? *reinterpret_cast<const uint4*>(kp_ + (size_t)e * 8) : make_uint4(0u, 0u, 0u, 0u); \
+    }                                                                                                     \
+    _Pragma("unroll") for (int gi = 0; gi < GB; ++gi) {                                                   \
+      const bf16* vp_ = vcache + ((size_t)page_ * G + min(g0 + gi, G - 1)) * dv * 64;                     \
+      _Pragma("unroll") for (int u = 0; u < VP; ++u) {                                                    \
+        const int e = threadIdx.x + u * SAM_WAVES * BLM_WAVE;                                             \
+        v_in[gi][u] = e < dv * 8 ? *reinterpret_cast<const uint4*>(vp_ + (size_t)e * 8) : make_uint4(0u, 0u, 0u, 0u); \
+      }                                                                                                   \
+    }                                                                                                     \
+  }
+  SAM_FETCH(blk_lo)
+  for (int pi = blk_lo; pi <= blk_hi; ++pi) {
+    const int key0 = pi * 64;
+    __syncthreads();                                                       // nobody reads the page before any more
+    _Pragma("unroll") for (int u = 0; u < KP; ++u) {
+      const int e = threadIdx.x + u * SAM_WAVES * BLM_WAVE;
+      if (e < 64 * k_pieces) {
+        const int row = e / k_pieces, piece = e - row * k_pieces;
+        *reinterpret_cast<uint4*>(k_sm + (size_t)row * krs + piece * 8) = k_in[u];
+      }
+    }
+    _Pragma("unroll") for (int gi = 0; gi < GB; ++gi) {
+      bf16* vs = v_sm + (size_t)gi * dv * vrs;
+      _Pragma("unroll") for (int u = 0; u < VP; ++u) {
+        const int e = threadIdx.x + u * SAM_WAVES * BLM_WAVE;
+        if (e < dv * 8) *reinterpret_cast<uint4*>(vs + (size_t)(e >> 3) * vrs + (e & 7) * 8) = v_in[gi][u];
+      }
+    }
+    __syncthreads();
+    if (pi < blk_hi) SAM_FETCH(pi + 1)                                     // travels while this page is worked on
+    if (pi < my_lo || pi > my_hi) continue;
+    float s[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bf16* krow = k_sm + (size_t)sa_key_of(t, c) * krs;
+      sa_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + kg * 8;
+        const uint4 kf = d < dk ? *reinterpret_cast<const uint4*>(krow + d) : make_uint4(0u, 0u, 0u, 0u);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sa_bf16x8, kf), __builtin_bit_cast(sa_bf16x8, qf[ks]),
+                                                      acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kj = key0 + sa_key_of(t, kg * 4 + r);
+        const bool seen = kj <= qpos && (window <= 0 || kj > qpos - window);
+        s[t][r] = seen ? acc[r] : -INFINITY;
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[t][r]);
+    mx = rows_max(mx);
+    const float m_new = fmaxf(m, mx * scale2);
+    const float corr = (m == m_new) ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        s[t][r] = (s[t][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale2, -m_new));
+    if (__any(m != m_new)) {
+#pragma unroll
+      for (int gi = 0; gi < GB; ++gi)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[gi][dt][r] *= corr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) l[r] *= corr;
+    }
+    m = m_new;
+    const bool tail = key0 + 63 > max_key;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 pf;
+      pf.x = f32x2_to_bf16x2_bits(s[2 * h][0], s[2 * h][1]);
+      pf.y = f32x2_to_bf16x2_bits(s[2 * h][2], s[2 * h][3]);
+      pf.z = f32x2_to_bf16x2_bits(s[2 * h + 1][0], s[2 * h + 1][1]);
+      pf.w = f32x2_to_bf16x2_bits(s[2 * h + 1][2], s[2 * h + 1][3]);
+      l = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          __builtin_bit_cast(sa_bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u)),
+          __builtin_bit_cast(sa_bf16x8, pf), l, 0, 0, 0);
+      const int keep = max_key - (key0 + h * 32 + kg * 8) + 1;
+#pragma unroll
+      for (int gi = 0; gi < GB; ++gi) {
+        if (g0 + gi < G) {
+          const bf16* vs = v_sm + (size_t)gi * dv * vrs;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const int row = dt * 16 + c;
+            uint4 va = row < dv ? *reinterpret_cast<const uint4*>(vs + (size_t)row * vrs + h * 32 + kg * 8) : make_uint4(0u, 0u, 0u, 0u);
+            if (tail) va = sa_keep_first(va, keep);
+            o[gi][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sa_bf16x8, va),
+                                                                __builtin_bit_cast(sa_bf16x8, pf), o[gi][dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (valid) {
+    const float inv = 1.0f / l[0];
+    float* arow = A + ((size_t)(t_first + tok) * H + head) * n_out * dv;
+#pragma unroll
+    for (int gi = 0; gi < GB; ++gi) {
+      const int cc = g0 + gi;
+      if (cc < G) {
+        float* og = arow + (size_t)(all_groups ? cc : 0) * dv;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int d = dt * 16 + kg * 4 + r;
+            if (d < dv) og[d] = o[gi][dt][r] * inv;
+          }
+      }
+    }
+  }
+}
+
+#undef SAM_FETCH
+
 // The pieces of a cut range added up, one block per column: maxima in base 2.  A piece that saw nothing and holds
 // no sink has sum 0, maximum -infinity and results of zeros, and gets weight 0.
 __global__ void __launch_bounds__(256)
@@ -519,6 +715,32 @@ __global__ void __launch_bounds__(256)
     for (int p = 0; p < n_splits; ++p) acc = fmaf(wgt[p], po[(size_t)p * n + d], acc);
     arow[d] = acc * inv_sum;
   }
+}
+
+#define SAM_STAGED_LDS (152 * 1024)
+#define SAM_DEVICES 64
+static bool g_sam_big_lds[SAM_DEVICES];
+#define SAM_ALL_CASES(X) X(2, 2) X(2, 3) X(2, 4) X(2, 8) X(4, 2) X(4, 3) X(4, 4) X(4, 8)
+// Once per device, outside any stream capture: lets the form that stages pages ask for more shared memory than a
+// kernel gets without asking.  Without it that form is not used.
+extern "C" int blm_sink_attn_mfma_init() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  BLM_REQUIRE(e == hipSuccess && dev >= 0, "sink_attn_mfma_init: hipGetDevice failed: %s", hipGetErrorString(e));
+  if (dev >= SAM_DEVICES) return 0;
+#define SAM_ATTR(KS, DT)                                                                                                  \
+  {                                                                                                                       \
+    const void* ks_[] = {(const void*)sink_attn_mfma_staged_kernel<KS, DT, 1>, (const void*)sink_attn_mfma_staged_kernel<KS, DT, 2>, \
+                         (const void*)sink_attn_mfma_staged_kernel<KS, DT, 4>};                                           \
+    for (const void* k : ks_) {                                                                                           \
+      e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, SAM_STAGED_LDS);                             \
+      BLM_REQUIRE(e == hipSuccess, "sink_attn_mfma_init: cannot raise the shared memory limit: %s", hipGetErrorString(e)); \
+    }                                                                                                                     \
+  }
+  SAM_ALL_CASES(SAM_ATTR)
+#undef SAM_ATTR
+  g_sam_big_lds[dev] = true;
+  return 0;
 }
 
 extern "C" int blm_sink_attn_mfma_supported(int dk, int dv) {
@@ -569,8 +791,31 @@ extern "C" int blm_sink_attn_mfma(const void* q, int ldq, void* out, float* A, c
     else if (dt == 4) SAM_GB(KS, 4);    \
     else SAM_GB(KS, 8);                 \
   } while (0)
-  if (ks == 2) SAM_DT(2);
-  else SAM_DT(4);
+  // prompts: the form that stages every page once per block of four tiles, where its pages fit the shared memory
+  const int Hg = H / G;
+  const size_t staged_lds = ((size_t)64 * (dk + 8) + (size_t)gb * dv * (64 + 8)) * sizeof(bf16);
+  int dev = -1;
+  const bool big = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < SAM_DEVICES && g_sam_big_lds[dev];
+  const bool staged = n_splits == 1 && (long long)max_new * Hg >= 64 && staged_lds <= (size_t)(big ? SAM_STAGED_LDS : 64 * 1024);
+  if (staged) {
+    const int blocks_per_seq = (int)((tiles + SAM_WAVES - 1) / SAM_WAVES);
+    dim3 sgrid((unsigned)((long long)B * G * blocks_per_seq), 1, grid.z);
+#undef SAM_CASE
+#define SAM_CASE(KS, DT, GB)                                                                                              \
+  hipLaunchKernelGGL((sink_attn_mfma_staged_kernel<KS, DT, GB>), sgrid, dim3(SAM_WAVES * BLM_WAVE), staged_lds, stream,    \
+                     (const bf16*)q, ldq, A, sinks, cu_seqlens, lens_after, block_table, table_width, (const bf16*)kcache, \
+                     (const bf16*)vcache, B, H, G, dk, dv, blocks_per_seq, scale2, window, all_groups)
+    if (ks == 2) SAM_DT(2);
+    else SAM_DT(4);
+  } else {
+#undef SAM_CASE
+#define SAM_CASE(KS, DT, GB)                                                                                              \
+  hipLaunchKernelGGL((sink_attn_mfma_kernel<KS, DT, GB>), grid, dim3(SAM_WAVES * BLM_WAVE), 0, stream, (const bf16*)q, ldq, A, \
+                     sinks, cu_seqlens, lens_after, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache, B, H, \
+                     G, dk, dv, (int)tiles, scale2, window, all_groups, n_splits, part_o, part_ml)
+    if (ks == 2) SAM_DT(2);
+    else SAM_DT(4);
+  }
 #undef SAM_DT
 #undef SAM_GB
 #undef SAM_CASE

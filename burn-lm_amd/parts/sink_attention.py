@@ -75,6 +75,7 @@ class SinkAttention(Mixer):
             and os.environ.get("BURN_LM_AMD_SINK_ATTENTION") != "generic"
         if self.on_matrix_cores:
             rt.ops.latent_attn_init(rt.device)     # the pieces' workspace, before any step is recorded
+            rt.ops.sink_attn_mfma_init(rt.device)  # likewise: the shared memory of the form that stages pages
         self.sinks = tensors[n["sink"]].float().contiguous() if sink else None
         self.talk = tensors[n["talk"]].float().contiguous() if talk else None
 
