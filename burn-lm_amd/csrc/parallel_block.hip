@@ -11,30 +11,39 @@
 __device__ __forceinline__ float pb_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 // ---------------------------------------------------------------------------------------
-// out_r[t][c] = n[t][c] + sum_k w_r[c][k] * n(t - taps + 1 + k)[c] for every reader r; rows before the step come
-// from hist [slots][taps-1][D] (oldest first; zeros in a fresh slot stand for "before the sequence").  n is the
-// float output of the norm; padding tokens (sequence -1) give zeros.
+// out_r[t][c] = n[t][c] + sum_k w_r[c][k] * n(t - taps + 1 + k)[c] for every reader r (one or two); rows before the
+// step come from hist [slots][taps-1][D] (oldest first; zeros in a fresh slot stand for "before the sequence").  n is
+// the float output of the norm; padding tokens (sequence -1) give zeros.
 // ---------------------------------------------------------------------------------------
 struct PbReaders {
   const float* w[PB_MAX_READERS];   // [D][taps]
   void* out[PB_MAX_READERS];        // [T][D]
 };
 
+// A block takes PB_TOKEN_TILE tokens x 256 channels (fewer tokens per block where a step brings few): a thread keeps its
+// channel's taps in registers and walks the tile's tokens, so that the taps are read once per tile and a row of n is
+// found in the nearest cache by the tokens behind it.
+#define PB_TOKEN_TILE 16
 template <typename TO>
-__global__ void input_conv_kernel(const float* __restrict__ n, const float* __restrict__ hist, PbReaders rd, int readers,
+__global__ void input_conv_kernel(const float* __restrict__ n, float* __restrict__ hist, PbReaders rd, int readers,
                                   int taps, const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
-                                  const int* __restrict__ seq_slots, int D) {
-  const int t = blockIdx.x;
-  const int b = token_seq[t];
-  const int c_first = blockIdx.y * blockDim.x + threadIdx.x, c_step = gridDim.y * blockDim.x;
-  if (b < 0) {
-    for (int c = c_first; c < D; c += c_step)
+                                  const int* __restrict__ seq_slots, int T, int D, int tile, int moves_history) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= D) return;
+  float w[2][PB_MAX_TAPS];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+#pragma unroll
+    for (int k = 0; k < PB_MAX_TAPS; ++k) w[r][k] = (r < readers && k < taps) ? rd.w[r][(size_t)c * taps + k] : 0.f;
+  const int t_end = min(T, (int)(blockIdx.x + 1) * tile);
+  for (int t = blockIdx.x * tile; t < t_end; ++t) {
+    const int b = token_seq[t];
+    if (b < 0) {
       for (int r = 0; r < readers; ++r) ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(0.f);
-    return;
-  }
-  const int start = cu_seqlens[b], slot = seq_slots[b];
-  const int off = t - start;
-  for (int c = c_first; c < D; c += c_step) {
+      continue;
+    }
+    const int start = cu_seqlens[b], slot = seq_slots[b];
+    const int off = t - start;
     float x[PB_MAX_TAPS];
 #pragma unroll
     for (int k = 0; k < PB_MAX_TAPS; ++k) {
@@ -44,13 +53,22 @@ __global__ void input_conv_kernel(const float* __restrict__ n, const float* __re
                         : (slot >= 0 ? hist[((size_t)slot * (taps - 1) + (taps - 1 + src)) * D + c] : 0.f);
       }
     }
-    for (int r = 0; r < readers; ++r) {
-      const float* w = rd.w[r] + (size_t)c * taps;
-      float a = 0.f;
+    const float cur = n[(size_t)t * D + c];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (r < readers) {
+        float a = 0.f;
+#pragma unroll
+        for (int k = 0; k < PB_MAX_TAPS; ++k)
+          if (k < taps) a = fmaf(w[r][k], x[k], a);
+        ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(cur + a);
+      }
+    }
+    // every sequence brings one token (decoding): this thread alone touches the channel's history, and has read it
+    if (moves_history && slot >= 0) {
 #pragma unroll
       for (int k = 0; k < PB_MAX_TAPS; ++k)
-        if (k < taps) a = fmaf(w[k], x[k], a);
-      ((TO*)rd.out[r])[(size_t)t * D + c] = from_float<TO>(n[(size_t)t * D + c] + a);
+        if (k < taps - 1) hist[((size_t)slot * (taps - 1) + k) * D + c] = x[k + 1];
     }
   }
 }
@@ -95,17 +113,20 @@ extern "C" int blm_input_conv(const float* n, float* hist, const float* w0, cons
   }
   // few tokens (decoding): a token's channels over several blocks, so that more than a handful of compute units work
   const int threads = 256;
-  const unsigned pieces = T >= 512 ? 1u : (unsigned)((D + threads - 1) / threads);
+  const unsigned pieces = (unsigned)((D + threads - 1) / threads);
+  const int tile = T >= 512 ? PB_TOKEN_TILE : 1;
+  const unsigned tiles = (unsigned)((T + tile - 1) / tile);
+  const int moves_history = (taps > 1 && T == B) ? 1 : 0;      // as many tokens as sequences: one each (a sequence brings at least one)
   if (out_dtype == BLM_F32)
-    hipLaunchKernelGGL(input_conv_kernel<float>, dim3(T, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
-                       cu_seqlens, seq_slots, D);
+    hipLaunchKernelGGL(input_conv_kernel<float>, dim3(tiles, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+                       cu_seqlens, seq_slots, T, D, tile, moves_history);
   else if (out_dtype == BLM_BF16)
-    hipLaunchKernelGGL(input_conv_kernel<bf16>, dim3(T, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
-                       cu_seqlens, seq_slots, D);
+    hipLaunchKernelGGL(input_conv_kernel<bf16>, dim3(tiles, pieces), dim3(threads), 0, stream, n, hist, rd, readers, taps, token_seq,
+                       cu_seqlens, seq_slots, T, D, tile, moves_history);
   else
     return blm_fail("input_conv: unsupported dtype %d", out_dtype);
   BLM_LAUNCH_CHECK("input_conv");
-  if (taps > 1) {
+  if (taps > 1 && !moves_history) {
     hipLaunchKernelGGL(input_history_kernel, dim3(B, (D + 255) / 256), dim3(256), 0, stream, n, taps, hist, cu_seqlens,
                        seq_slots, D);
     BLM_LAUNCH_CHECK("input_history");

@@ -362,6 +362,20 @@ __global__ void __launch_bounds__(SAM_WAVES* BLM_WAVE)
     const int page = bt[pi];
     const int key0 = pi * 64;
     const bf16* kp = kcache + ((size_t)page * G + kvh) * 64 * dk;
+    // one key-value head per wavefront (steps of few tiles): its value fragments are asked for here, in front of the
+    // scores, so that a page costs one trip to memory and not two in a row
+    uint4 v_early[GB == 1 ? 2 : 1][GB == 1 ? DT : 1];
+    if (GB == 1 && g0 < G) {
+      const bf16* vp = vcache + ((size_t)page * G + g0) * dv * 64;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const int row = dt * 16 + c;
+          v_early[GB == 1 ? h : 0][GB == 1 ? dt : 0] =
+              row < dv ? *reinterpret_cast<const uint4*>(vp + (size_t)row * 64 + h * 32 + kg * 8) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
     float s[4][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -429,7 +443,9 @@ __global__ void __launch_bounds__(SAM_WAVES* BLM_WAVE)
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
             const int row = dt * 16 + c;
-            uint4 va = row < dv ? *reinterpret_cast<const uint4*>(vp + (size_t)row * 64 + h * 32 + kg * 8) : make_uint4(0u, 0u, 0u, 0u);
+            uint4 va;
+            if (GB == 1) va = v_early[GB == 1 ? h : 0][GB == 1 ? dt : 0];
+            else va = row < dv ? *reinterpret_cast<const uint4*>(vp + (size_t)row * 64 + h * 32 + kg * 8) : make_uint4(0u, 0u, 0u, 0u);
             if (tail) va = sa_keep_first(va, keep);
             o[gi][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sa_bf16x8, va),
                                                                 __builtin_bit_cast(sa_bf16x8, pf), o[gi][dt], 0, 0, 0);
