@@ -382,6 +382,68 @@ def test_sizes_that_are_no_multiples_of_eight(tmp_path, dtype):
     rows.check()
 
 
+def drawn_config(seed):
+    """A configuration drawn from the seed: two to five layers of either mixer in any order, borrowers of earlier
+    attention layers with head counts, windows and scales of their own, any feed-forward or none, sizes that are and are
+    not multiples of eight, one tap and several."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *a: a[int(rng.integers(0, len(a)))]
+    layers, lenders = [], []
+    for i in range(int(rng.integers(2, 6))):
+        kind = pick("dense", "moe", None)
+        if kind == "dense":
+            mlp = dict(kind="dense", ff=pick(24, 64, 100), limit=pick(0.5, 1.0, 3.0))
+        elif kind == "moe":
+            E = int(rng.integers(2, 9))
+            mlp = dict(kind="moe", router=dict(experts=E, top=int(rng.integers(1, E + 1))), expert=dict(ff=pick(8, 16, 40)))
+            if rng.random() < 0.6:
+                mlp["shared"] = dict(ff=pick(8, 32, 48))
+        else:
+            mlp = None
+        if rng.random() < 0.4:
+            mixer = dict(heads=int(rng.integers(1, 5)), dim=pick(8, 16, 24, 48, 5), vdim=pick(8, 16, 32, 20, 3), tau=pick(1.0, 4.0, 16.0))
+            layers.append(dict(type="gla", mixer=mixer, mlp=mlp))
+            continue
+        if lenders and rng.random() < 0.5:
+            j = pick(*lenders)
+            mixer = dict(layers[j]["mixer"], kv_from=j, mask=dict(size=pick(1, 3, 17, 64, 65, 100, 300)), scale=pick(0.1, 0.25, 0.5))
+            mixer["heads"] = mixer["kv_heads"] * int(rng.integers(1, 5))
+        else:
+            G, dk = int(rng.integers(1, 5)), pick(8, 16, 24, 32, 48, 64, 12, 6)
+            mixer = dict(heads=G * int(rng.integers(1, 5)), kv_heads=G, dim=dk, vdim=pick(8, 16, 24, 48, 64, 10, 72), scale=pick(0.1, 0.25, 0.5),
+                         mask=dict(size=pick(1, 3, 17, 64, 65, 100, 300)),
+                         rot=dict(base=pick(100.0, 10000.0, 5e5), dims=pick(*[d for d in (2, 4, 6, 8, 12, 16, 24, 32, 48, 64) if d <= dk])))
+            lenders.append(i)
+        layers.append(dict(type="attention", mixer=mixer, mlp=mlp))
+    return config(layers, width=pick(40, 64, 96, 128, 72), vocab=pick(50, 101, 257), taps=int(rng.integers(1, 6)), side=pick(3, 8, 16),
+                  scale=pick(0.5, 1.0, 2.0), eps=pick(1e-5, 1e-6))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+def test_drawn_configurations(tmp_path, seed, dtype):
+    """Unequal prompts in one step, then 32 tokens one by one, for configurations nobody chose by hand."""
+    cfg = drawn_config(seed)
+    w = make_weights(cfg, 100 + seed, rank=(3, 8, 16)[seed % 3])
+    eng = engine_for(tmp_path, cfg, w, dtype, max_tokens=2048)
+    reqs = [tokens_of(cfg, 7 + seed + i, n) for i, n in enumerate((330, 9, 140))]
+    want = [P.forward(cfg, w, r) for r in reqs]
+    rows = Rows(dtype)
+    slots = [eng.open() for _ in reqs]
+    cut = [max(1, len(r) - 32) for r in reqs]
+    got = eng.step([(s, r[:c], list(range(c))) for s, r, c in zip(slots, reqs, cut)]).double().cpu().numpy()
+    o = 0
+    for i, c in enumerate(cut):
+        rows.add(got[o:o + c], want[i][:c], ("prompt", i))
+        o += c
+    for k in range(32):
+        live = [i for i in range(len(reqs)) if cut[i] + k < len(reqs[i])]
+        got = eng.step([(slots[i], [reqs[i][cut[i] + k]], [0]) for i in live]).double().cpu().numpy()
+        rows.add(got, np.stack([want[i][cut[i] + k] for i in live]), k)
+    rows.check()
+
+
 class _Step:
     """The index arrays that the attention kernels read, for sequences laid out by hand."""
 
