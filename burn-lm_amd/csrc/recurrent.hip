@@ -1,13 +1,15 @@
 // Recurrent mixers whose state is a matrix [key channels][value channels] per head and sequence, kept in
 // float in the cache's state tensors: a linear recurrence with one gate that shares a channel between its old state and
-// the new value (HGRN2), and a delta rule with one decay per key channel.  The columns of the state (one per value
+// the new value (HGRN2), a delta rule with one decay per key channel, and gated linear attention (a decay per key
+// channel, every token's key and value added as an outer product).  The columns of the state (one per value
 // channel) never meet: each needs only its own value and what the token brings per key channel (gates, keys,
 // queries).  So one wavefront walks the tokens of one (sequence, head) for 16 columns (or 4): the 4 (or 16) lanes of a
 // column each keep a share of its rows in registers and add their parts of a dot product with a few cross-lane
 // steps, and nothing waits for another wavefront.  What a token brings per key channel is
 // computed by the wavefront into its own piece of shared memory, from inputs it loaded one token ahead.  The
 // results go out unnormalised in float; a second kernel takes the root mean square over each head's value
-// lanes, the weight and (delta rule) the output gate.  The same kernels serve prompts and decoding.
+// lanes, the weight and (delta rule, gated linear attention) the output gate.  The same kernels serve prompts and
+// decoding; gated linear attention also cuts a prompt into segments that several wavefronts walk at once.
 //
 // Also here: the short causal convolution in front of the delta rule with its per-sequence history.
 #include "common.h"
